@@ -1,0 +1,133 @@
+"""Build and load ``libconnect6_amd.so`` (hand-written HIP for gfx950) via ctypes.
+
+The library is the only compute backend of this package: there is no PyTorch
+or CPU fallback.  ``load()`` raises if the shared object is missing.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+from pathlib import Path
+
+_PKG = Path(__file__).resolve().parent
+_CSRC = _PKG / "csrc"
+_LIBDIR = _PKG / "lib"
+_SO = _LIBDIR / "libconnect6_amd.so"
+_SOURCES = ("c6_forward.hip", "c6_tail.hip", "c6_api.hip")
+
+# arithmetic modes (include/connect6_amd.h)
+PREC_F32, PREC_BF16, PREC_F16, PREC_BF16X2 = 0, 1, 2, 3
+PREC_BY_NAME = {"fp32": PREC_F32, "bf16": PREC_BF16, "fp16": PREC_F16, "bf16x2": PREC_BF16X2}
+DT_F32, DT_BF16, DT_F16 = 0, 1, 2
+MASK_NONE, MASK_INPUT, MASK_LEGAL = 0, 1, 2
+
+# every symbol include/connect6_amd.h declares
+EXPORTS = (
+    "c6_version",
+    "c6_last_error",
+    "c6_packed_bytes",
+    "c6_pack_weights",
+    "c6_forward",
+    "c6_mask_logits",
+    "c6_softmax_sample",
+    "c6_d4_expand",
+    "c6_d4_reduce",
+)
+
+
+class C6Error(RuntimeError):
+    pass
+
+
+def build(verbose: bool = False) -> Path:
+    """Compile the HIP sources for gfx950 into ``lib/libconnect6_amd.so``."""
+    _LIBDIR.mkdir(exist_ok=True)
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    cmd = [
+        hipcc, "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+        # packed-fp32 VALU forms are disabled for every kernel in this library
+        "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+        "-Wall", "-Wno-unused-function",
+        "-o", str(_SO),
+    ] + [str(_CSRC / s) for s in _SOURCES]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if verbose or proc.returncode != 0:
+        print(proc.stdout)
+        print(proc.stderr)
+    if proc.returncode != 0:
+        raise C6Error(f"hipcc failed ({proc.returncode}):\n{proc.stderr[-4000:]}")
+    return _SO
+
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not _SO.exists():
+        raise C6Error(
+            f"{_SO} is missing: build it with connect6_amd.build() "
+            "(hipcc --offload-arch=gfx950); there is no fallback path"
+        )
+    lib = ctypes.CDLL(str(_SO))
+    vp, i32, i64, f32 = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_float
+    lib.c6_version.restype = i32
+    lib.c6_version.argtypes = []
+    lib.c6_last_error.restype = ctypes.c_char_p
+    lib.c6_last_error.argtypes = []
+    lib.c6_packed_bytes.restype = i32
+    lib.c6_packed_bytes.argtypes = [i32, ctypes.POINTER(ctypes.c_size_t)]
+    lib.c6_pack_weights.restype = i32
+    lib.c6_pack_weights.argtypes = [ctypes.POINTER(vp), ctypes.POINTER(vp), vp, vp, vp, vp, i32, vp, vp]
+    lib.c6_forward.restype = i32
+    lib.c6_forward.argtypes = [vp, i32, i64, i64, vp, ctypes.c_size_t, i32, vp, vp, i32, vp, f32,
+                               vp, f32, vp, vp, vp]
+    lib.c6_mask_logits.restype = i32
+    lib.c6_mask_logits.argtypes = [vp, vp, i32, i64, ctypes.c_uint32, vp, vp]
+    lib.c6_softmax_sample.restype = i32
+    lib.c6_softmax_sample.argtypes = [vp, vp, vp, f32, i64, vp, vp, vp]
+    lib.c6_d4_expand.restype = i32
+    lib.c6_d4_expand.argtypes = [vp, i32, i64, vp, vp]
+    lib.c6_d4_reduce.restype = i32
+    lib.c6_d4_reduce.argtypes = [vp, vp, i64, vp, vp, vp]
+    _lib = lib
+    return lib
+
+
+def check(rc: int, what: str) -> None:
+    """Map a library return code to the exception the reference would raise:
+    bad shapes/dtypes are ValueError (connect6/model.py:98-102), anything the
+    device reports is RuntimeError."""
+    if rc == 0:
+        return
+    msg = load().c6_last_error().decode("utf-8", "replace")
+    if rc == -1:
+        raise ValueError(f"{what}: {msg}")
+    raise C6Error(f"{what}: {msg} (code {rc})")
+
+
+def packed_bytes(prec: int) -> int:
+    n = ctypes.c_size_t(0)
+    check(load().c6_packed_bytes(prec, ctypes.byref(n)), "c6_packed_bytes")
+    return int(n.value)
+
+
+def torch_dtype_code(dtype) -> int:
+    import torch
+
+    if dtype == torch.float32:
+        return DT_F32
+    if dtype == torch.bfloat16:
+        return DT_BF16
+    if dtype == torch.float16:
+        return DT_F16
+    raise ValueError(f"unsupported tensor dtype {dtype}; expected float32, bfloat16 or float16")
+
+
+def stream_ptr(device) -> int:
+    import torch
+
+    return int(torch.cuda.current_stream(device).cuda_stream)

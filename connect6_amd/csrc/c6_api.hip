@@ -1,0 +1,203 @@
+// extern "C" boundary of libconnect6_amd.so: argument validation and dispatch.
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "c6_common.h"
+
+namespace c6 {
+
+static thread_local char g_error[512] = "";
+
+void set_error(const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+}
+
+int dispatch_pack(int prec, const PackParams &pp, hipStream_t st);
+int dispatch_forward(int prec, const FwdParams &fp, hipStream_t st);
+size_t packed_bytes(int prec);
+int launch_mask(const void *, const uint8_t *, int, long long, uint32_t, void *, hipStream_t);
+int launch_sample(const float *, const uint8_t *, const float *, float, long long, long long *,
+                  float *, hipStream_t);
+int launch_d4_expand(const void *, int, long long, void *, hipStream_t);
+int launch_d4_reduce(const float *, const float *, long long, float *, float *, hipStream_t);
+
+static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+static int elem_bytes(int dt) { return dt == C6_DT_F32 ? 4 : ((dt == C6_DT_BF16 || dt == C6_DT_F16) ? 2 : 0); }
+static bool valid_prec(int p) { return p >= C6_PREC_F32 && p <= C6_PREC_BF16X2; }
+
+}  // namespace c6
+
+using namespace c6;
+
+extern "C" {
+
+int c6_version(void) { return 1; }
+
+const char *c6_last_error(void) { return g_error; }
+
+int c6_packed_bytes(int prec, size_t *bytes) {
+  if (!valid_prec(prec) || bytes == nullptr) {
+    set_error("c6_packed_bytes: bad precision mode %d or null output", prec);
+    return C6_EINVAL;
+  }
+  *bytes = packed_bytes(prec);
+  return C6_OK;
+}
+
+int c6_pack_weights(const float *const *conv_w, const float *const *conv_b, const float *pol_w,
+                    const float *pol_b, const float *val_w, const float *val_b, int prec,
+                    void *packed, void *stream) {
+  if (!valid_prec(prec)) {
+    set_error("c6_pack_weights: unknown precision mode %d", prec);
+    return C6_EINVAL;
+  }
+  if (conv_w == nullptr || pol_w == nullptr || packed == nullptr) {
+    set_error("c6_pack_weights: conv_w, pol_w and packed must not be null");
+    return C6_EINVAL;
+  }
+  if (!aligned16(packed)) {
+    set_error("c6_pack_weights: packed buffer must be 16-byte aligned");
+    return C6_EINVAL;
+  }
+  PackParams pp;
+  for (int i = 0; i < 8; ++i) {
+    if (conv_w[i] == nullptr) {
+      set_error("c6_pack_weights: conv_w[%d] is null", i);
+      return C6_EINVAL;
+    }
+    pp.conv_w[i] = conv_w[i];
+    pp.conv_b[i] = conv_b ? conv_b[i] : nullptr;
+  }
+  pp.pol_w = pol_w;
+  pp.pol_b = pol_b;
+  pp.val_w = val_w;
+  pp.val_b = val_b;
+  pp.packed = static_cast<unsigned char *>(packed);
+  return dispatch_pack(prec, pp, static_cast<hipStream_t>(stream));
+}
+
+int c6_forward(const void *x, int x_dtype, int64_t groups, int64_t boards_per_group,
+               const void *packed, size_t packed_stride, int prec, float *logits, float *value,
+               int mask_mode, const uint8_t *legal, float fill, const float *u, float temperature,
+               int64_t *actions, float *logprob, void *stream) {
+  if (!valid_prec(prec)) {
+    set_error("c6_forward: unknown precision mode %d", prec);
+    return C6_EINVAL;
+  }
+  if (elem_bytes(x_dtype) == 0) {
+    set_error("c6_forward: unknown input element type %d", x_dtype);
+    return C6_EINVAL;
+  }
+  if (groups < 1 || boards_per_group < 0) {
+    set_error("c6_forward: groups=%lld boards_per_group=%lld out of range", (long long)groups,
+              (long long)boards_per_group);
+    return C6_EINVAL;
+  }
+  if (boards_per_group == 0) return C6_OK;  // empty batch: nothing to do
+  if (x == nullptr || packed == nullptr) {
+    set_error("c6_forward: x and packed must not be null");
+    return C6_EINVAL;
+  }
+  if (!aligned16(packed) || (packed_stride & 15u) != 0 ||
+      (groups > 1 && packed_stride < packed_bytes(prec))) {
+    set_error("c6_forward: packed weights must be 16-byte aligned with stride >= one set");
+    return C6_EINVAL;
+  }
+  if (mask_mode < C6_MASK_NONE || mask_mode > C6_MASK_LEGAL ||
+      (mask_mode == C6_MASK_LEGAL && legal == nullptr)) {
+    set_error("c6_forward: bad mask_mode %d (legal mask %s)", mask_mode, legal ? "given" : "missing");
+    return C6_EINVAL;
+  }
+  if (actions != nullptr && u == nullptr) {
+    set_error("c6_forward: sampling needs the uniform draws u");
+    return C6_EINVAL;
+  }
+  FwdParams fp;
+  fp.x = x;
+  fp.x_dtype = x_dtype;
+  fp.total_boards = groups * boards_per_group;
+  fp.boards_per_group = boards_per_group;
+  fp.packed = static_cast<const unsigned char *>(packed);
+  fp.packed_stride = packed_stride;
+  fp.logits = logits;
+  fp.value = value;
+  fp.mask_mode = mask_mode;
+  fp.legal = legal;
+  fp.fill = fill;
+  fp.u = u;
+  fp.inv_temperature = 1.0f / (temperature > 1e-4f ? temperature : 1e-4f);
+  fp.actions = reinterpret_cast<long long *>(actions);
+  fp.logprob = logprob;
+  return dispatch_forward(prec, fp, static_cast<hipStream_t>(stream));
+}
+
+int c6_mask_logits(const void *logits, const uint8_t *legal, int dtype, int64_t batch,
+                   uint32_t fill_bits, void *out, void *stream) {
+  const int eb = elem_bytes(dtype);
+  if (eb == 0 || batch < 0) {
+    set_error("c6_mask_logits: bad dtype %d or batch %lld", dtype, (long long)batch);
+    return C6_EINVAL;
+  }
+  if (batch == 0) return C6_OK;
+  if (logits == nullptr || legal == nullptr || out == nullptr) {
+    set_error("c6_mask_logits: null pointer");
+    return C6_EINVAL;
+  }
+  if (!aligned16(logits) || !aligned16(out) || (reinterpret_cast<uintptr_t>(legal) & 7u)) {
+    set_error("c6_mask_logits: logits/out must be 16-byte and legal 8-byte aligned");
+    return C6_EINVAL;
+  }
+  return launch_mask(logits, legal, eb, (long long)batch * C6_ACTIONS, fill_bits, out,
+                     static_cast<hipStream_t>(stream));
+}
+
+int c6_softmax_sample(const float *logits, const uint8_t *legal, const float *u, float temperature,
+                      int64_t batch, int64_t *actions, float *logprob, void *stream) {
+  if (batch < 0) {
+    set_error("c6_softmax_sample: negative batch");
+    return C6_EINVAL;
+  }
+  if (batch == 0) return C6_OK;
+  if (logits == nullptr || u == nullptr || actions == nullptr) {
+    set_error("c6_softmax_sample: logits, u and actions must not be null");
+    return C6_EINVAL;
+  }
+  const float inv_t = 1.0f / (temperature > 1e-4f ? temperature : 1e-4f);
+  return launch_sample(logits, legal, u, inv_t, batch, reinterpret_cast<long long *>(actions),
+                       logprob, static_cast<hipStream_t>(stream));
+}
+
+int c6_d4_expand(const void *x, int dtype, int64_t batch, void *out, void *stream) {
+  const int eb = elem_bytes(dtype);
+  if (eb == 0 || batch < 0) {
+    set_error("c6_d4_expand: bad dtype %d or batch %lld", dtype, (long long)batch);
+    return C6_EINVAL;
+  }
+  if (batch == 0) return C6_OK;
+  if (x == nullptr || out == nullptr) {
+    set_error("c6_d4_expand: null pointer");
+    return C6_EINVAL;
+  }
+  return launch_d4_expand(x, eb, batch, out, static_cast<hipStream_t>(stream));
+}
+
+int c6_d4_reduce(const float *view_logits, const float *view_values, int64_t batch, float *logits,
+                 float *values, void *stream) {
+  if (batch < 0) {
+    set_error("c6_d4_reduce: negative batch");
+    return C6_EINVAL;
+  }
+  if (batch == 0) return C6_OK;
+  if (view_logits == nullptr || logits == nullptr || (values != nullptr && view_values == nullptr)) {
+    set_error("c6_d4_reduce: null pointer");
+    return C6_EINVAL;
+  }
+  return launch_d4_reduce(view_logits, view_values, batch, logits, values,
+                          static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,144 @@
+// Shared definitions of the connect6_amd HIP sources (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+
+#include "../../include/connect6_amd.h"
+
+namespace c6 {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+// ---- network geometry (default architecture, connect6/model.py:22-24) ----
+constexpr int kBoard = 19;
+constexpr int kPix = 361;
+constexpr int kLayers = 8;
+constexpr int kK1 = 23;                                   // first-layer kernel
+constexpr int kCinArr[8] = {3, 32, 32, 64, 64, 64, 96, 96};
+constexpr int kCoutArr[8] = {32, 32, 64, 64, 64, 96, 96, 96};
+constexpr int kBiasTotal = 32 + 32 + 64 + 64 + 64 + 96 + 96 + 96;  // 544
+constexpr int kHeadC = 96;
+
+// ---- on-chip activation tile -------------------------------------------
+// One board lives in LDS as 421 positions x 96 channel slots, channel-last.
+// Position index of square (r,c) is (r+1)*20 + (c+1): rows are 20 apart so a
+// single zero column serves as right pad of one row and left pad of the next;
+// rows 0 and 20 (+ position 420) are the top/bottom pad.  A 3x3 tap is then
+// the constant position offset (ky-1)*20 + (kx-1).
+constexpr int kPitch = 20;
+constexpr int kPos = 421;
+constexpr int kChSlots = 96;
+
+// ---- first layer (23x23 on 3 planes, K = 3*529 lowered densely) -----------
+// K is ordered (ky, plane, kx) with kx padded 23 -> 24; the 69 (ky,plane) rows
+// are padded to 70 and split in two halves of 35: MFMA lane-half h contracts
+// rows [35h, 35h+35).  The zero-padded 41-wide halo is held in E = 16/sizeof(T)
+// copies, copy s shifted left by s elements, so that every 16-byte operand
+// fragment (E consecutive kx of one row) is 16-byte aligned for every column.
+constexpr int kL1RowsHalf = 35;
+constexpr int kL1RowPitch = 40;   // elements per halo row in a shifted copy
+constexpr int kL1CopyRows = 124;  // 41*3 rows + 1 zero row read by the padded K tail
+
+// MFMA tiling: 256 threads = 4 waves; wave w owns pixels [96w, 96w+96) as three
+// 32-pixel column tiles, and all Cout/32 row tiles of output channels.
+constexpr int kThreads = 256;
+constexpr int kWaves = 4;
+constexpr int kPixPerWave = 96;
+
+constexpr int kRing = 6;          // weight-fragment prefetch depth (k-steps)
+constexpr int kOverreadFrags = 8 * 3;  // zero frags after the last layer (prefetch may over-read)
+
+// precision policies ----------------------------------------------------------
+struct PrecF32 {
+  static constexpr int ID = C6_PREC_F32;
+  static constexpr int EB = 4;        // bytes per element
+  static constexpr int SPLIT = 0;
+};
+struct PrecBF16 {
+  static constexpr int ID = C6_PREC_BF16;
+  static constexpr int EB = 2;
+  static constexpr int SPLIT = 0;
+};
+struct PrecF16 {
+  static constexpr int ID = C6_PREC_F16;
+  static constexpr int EB = 2;
+  static constexpr int SPLIT = 0;
+};
+struct PrecBF16X2 {
+  static constexpr int ID = C6_PREC_BF16X2;
+  static constexpr int EB = 2;
+  static constexpr int SPLIT = 1;     // activations stored as hi plane + lo plane
+};
+
+template <class P> struct Geo {
+  static constexpr int EB = P::EB;
+  static constexpr int E = 16 / EB;                 // elements per 16-byte fragment lane
+  static constexpr int KSTEP = 2 * E;               // K elements contracted per fragment pair
+  static constexpr int PLANE = kChSlots * EB;       // bytes of one precision plane of a position
+  static constexpr int PIXB = PLANE * (P::SPLIT ? 2 : 1);  // bytes per position
+  static constexpr int ACT_BYTES = kPos * PIXB;
+  static constexpr int CPR = 24 / E;                // fragments per first-layer K row
+  static constexpr int STEPS1 = kL1RowsHalf * CPR;  // first-layer k-steps
+  static constexpr int COPY_BYTES = kL1CopyRows * kL1RowPitch * EB;
+  static constexpr int COPIES_BYTES = E * COPY_BYTES;
+  static constexpr int BUF_BYTES = ACT_BYTES > COPIES_BYTES ? ACT_BYTES : COPIES_BYTES;
+  // LDS map: [activation tile | first-layer copies] [occupancy 384] [logits 361 f32] [partials]
+  static constexpr int OCC_OFF = (BUF_BYTES + 15) & ~15;
+  static constexpr int LGT_OFF = OCC_OFF + 384;
+  static constexpr int RED_OFF = LGT_OFF + 1456;
+  static constexpr int LDS_BYTES = RED_OFF + 64;
+
+  static constexpr int layer_steps(int l) { return l == 0 ? STEPS1 : 9 * kCinArr[l] / KSTEP; }
+  static constexpr int layer_frags(int l) { return layer_steps(l) * (kCoutArr[l] / 32); }
+  static constexpr int frag_offset(int l) {  // in 1 KiB fragments
+    int s = 0;
+    for (int i = 0; i < l; ++i) s += layer_frags(i);
+    return s;
+  }
+  static constexpr int TOTAL_FRAGS = frag_offset(8) + kOverreadFrags;
+  static constexpr size_t TAIL_OFF = (size_t)TOTAL_FRAGS * 1024;  // fp32 tail: biases, heads
+  // tail floats: bias[544] polw[96] valw[96] polb valb (+pad)
+  static constexpr int TAIL_FLOATS = kBiasTotal + 2 * kHeadC + 4;
+  static constexpr size_t PACKED_BYTES = TAIL_OFF + (size_t)TAIL_FLOATS * 4;
+};
+
+constexpr int bias_offset(int l) {
+  int s = 0;
+  for (int i = 0; i < l; ++i) s += kCoutArr[i];
+  return s;
+}
+
+struct FwdParams {
+  const void *x;
+  int x_dtype;
+  long long total_boards;
+  long long boards_per_group;
+  const unsigned char *packed;
+  size_t packed_stride;
+  float *logits;
+  float *value;
+  int mask_mode;
+  const uint8_t *legal;
+  float fill;
+  const float *u;
+  float inv_temperature;
+  long long *actions;
+  float *logprob;
+};
+
+struct PackParams {
+  const float *conv_w[8];
+  const float *conv_b[8];
+  const float *pol_w, *pol_b, *val_w, *val_b;
+  unsigned char *packed;
+};
+
+void set_error(const char *fmt, ...);
+
+}  // namespace c6

@@ -1,0 +1,558 @@
+// Fused forward of the Connect6 policy/value CNN for gfx950 (MI355X).
+//
+// One workgroup (4 waves) carries one board through all eight convolutions and
+// both heads without leaving the CU: the 19x19xC activation tile stays in LDS
+// (channel-last, written in place after a barrier because every wave keeps its
+// whole output tile in MFMA accumulators), weights stream from L2 straight
+// into registers in MFMA-fragment order, and the grid is persistent over
+// boards.  Replaces PolicyValueNet.forward (connect6/model.py:96-111 of the
+// reference) and, with several weight sets, HistoricalPolicyEnsemble
+// .forward_grouped (connect6/history.py:276-303).
+//
+// Implicit GEMM orientation: D[cout, pixel] += W[cout, k] * X[k, pixel], so an
+// accumulator lane holds ONE pixel and 16 channels -- the epilogue writes four
+// consecutive channels per store and the 1x1 heads reduce mostly inside a lane.
+#include "c6_common.h"
+#include "c6_device.h"
+
+namespace c6 {
+
+// ------------------------------------------------------------------------
+// precision-specific primitives
+// ------------------------------------------------------------------------
+template <class P> __device__ __forceinline__ void mma(const v4i &a, const v4i &b, f32x16 &c);
+
+template <> __device__ __forceinline__ void mma<PrecBF16>(const v4i &a, const v4i &b, f32x16 &c) {
+  c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                              __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+template <> __device__ __forceinline__ void mma<PrecBF16X2>(const v4i &a, const v4i &b, f32x16 &c) {
+  mma<PrecBF16>(a, b, c);
+}
+template <> __device__ __forceinline__ void mma<PrecF16>(const v4i &a, const v4i &b, f32x16 &c) {
+  c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
+                                             __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+template <> __device__ __forceinline__ void mma<PrecF32>(const v4i &a, const v4i &b, f32x16 &c) {
+  const f32x4 af = __builtin_bit_cast(f32x4, a);
+  const f32x4 bf = __builtin_bit_cast(f32x4, b);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) c = __builtin_amdgcn_mfma_f32_32x32x2f32(af[e], bf[e], c, 0, 0, 0);
+}
+
+template <class P> __device__ __forceinline__ unsigned short bits16(float v);
+template <> __device__ __forceinline__ unsigned short bits16<PrecBF16>(float v) {
+  return __builtin_bit_cast(unsigned short, (__bf16)v);
+}
+template <> __device__ __forceinline__ unsigned short bits16<PrecBF16X2>(float v) {
+  return __builtin_bit_cast(unsigned short, (__bf16)v);
+}
+template <> __device__ __forceinline__ unsigned short bits16<PrecF16>(float v) {
+  return __builtin_bit_cast(unsigned short, (_Float16)v);
+}
+template <> __device__ __forceinline__ unsigned short bits16<PrecF32>(float) { return 0; }
+
+template <class P> __device__ __forceinline__ float from_bits16(unsigned short b);
+template <> __device__ __forceinline__ float from_bits16<PrecBF16X2>(unsigned short b) {
+  return __builtin_bit_cast(float, (unsigned)b << 16);
+}
+
+// store four consecutive channels of one position (dst already swizzled)
+template <class P> __device__ __forceinline__ void store4(unsigned char *dst, const float (&v)[4]) {
+  if constexpr (P::EB == 4) {
+    f32x4 o = {v[0], v[1], v[2], v[3]};
+    *reinterpret_cast<f32x4 *>(dst) = o;
+  } else {
+    v2i o;
+    o[0] = (int)((unsigned)bits16<P>(v[0]) | ((unsigned)bits16<P>(v[1]) << 16));
+    o[1] = (int)((unsigned)bits16<P>(v[2]) | ((unsigned)bits16<P>(v[3]) << 16));
+    *reinterpret_cast<v2i *>(dst) = o;
+    if constexpr (P::SPLIT) {
+      float r[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) r[e] = v[e] - from_bits16<P>(bits16<P>(v[e]));
+      v2i q;
+      q[0] = (int)((unsigned)bits16<P>(r[0]) | ((unsigned)bits16<P>(r[1]) << 16));
+      q[1] = (int)((unsigned)bits16<P>(r[2]) | ((unsigned)bits16<P>(r[3]) << 16));
+      *reinterpret_cast<v2i *>(dst + Geo<P>::PLANE) = q;
+    }
+  }
+}
+
+template <class P> __device__ __forceinline__ float silu(float v) {
+  if constexpr (P::EB == 4) {
+    return v / (1.0f + expf(-v));
+  } else {
+    return v * __builtin_amdgcn_rcpf(1.0f + __expf(-v));
+  }
+}
+
+__device__ __forceinline__ float load_x(const void *x, int dt, size_t i) {
+  if (dt == C6_DT_F32) return reinterpret_cast<const float *>(x)[i];
+  const unsigned short b = reinterpret_cast<const unsigned short *>(x)[i];
+  if (dt == C6_DT_BF16) return __builtin_bit_cast(float, (unsigned)b << 16);
+  return (float)__builtin_bit_cast(_Float16, b);
+}
+
+// ------------------------------------------------------------------------
+// first layer: 23x23 on 3 planes, K = (ky, plane, kx24) split over lane halves
+// ------------------------------------------------------------------------
+template <class P>
+__device__ __forceinline__ void conv1_accumulate(const unsigned char *smem,
+                                                 const v4i *__restrict__ wl,
+                                                 const int (&l1base)[3], f32x16 (&acc)[1][3]) {
+  using G = Geo<P>;
+  constexpr int CPR = G::CPR;
+  constexpr int ROWB = kL1RowPitch * G::EB;
+  constexpr int ROWS_BODY = (CPR == 3) ? 7 : 1;
+  constexpr int U = ROWS_BODY * CPR;
+  constexpr int D = (CPR == 3) ? 7 : 6;
+  constexpr int ITERS = kL1RowsHalf / ROWS_BODY;
+  static_assert(U % D == 0 && ITERS * ROWS_BODY == kL1RowsHalf, "first-layer pipeline shape");
+
+  v4i ring[D];
+#pragma unroll
+  for (int d = 0; d < D; ++d) ring[d] = wl[d * 64];
+#pragma unroll 1
+  for (int it = 0; it < ITERS; ++it) {
+    const int adv = it * ROWS_BODY * ROWB;
+    const v4i *wn = wl + (size_t)(it * U + D) * 64;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int off = (u / CPR) * ROWB + (u % CPR) * 16;
+      v4i b[3];
+#pragma unroll
+      for (int j = 0; j < 3; ++j) b[j] = *reinterpret_cast<const v4i *>(smem + l1base[j] + adv + off);
+#pragma unroll
+      for (int j = 0; j < 3; ++j) mma<P>(ring[u % D], b[j], acc[0][j]);
+      ring[u % D] = wn[u * 64];  // prefetch k-step (it*U + u + D); the tail over-reads zero frags
+    }
+  }
+}
+
+// ------------------------------------------------------------------------
+// 3x3 layers: K = (tap, cin), cin fastest; taps are constant position offsets
+// ------------------------------------------------------------------------
+template <class P, int CIN, int COUT>
+__device__ __forceinline__ void conv3_accumulate(const unsigned char *smem,
+                                                 const v4i *__restrict__ wl, const int (&ci)[3],
+                                                 int h, f32x16 (&acc)[COUT / 32][3]) {
+  using G = Geo<P>;
+  constexpr int NT = COUT / 32;
+  constexpr int KC = CIN / G::KSTEP;
+  constexpr int U = 3 * KC;  // k-steps of one kernel row
+  constexpr int D = kRing;
+  static_assert(U % D == 0, "ring depth must divide the k-steps of a kernel row");
+
+  v4i ring[D][NT];
+#pragma unroll
+  for (int d = 0; d < D; ++d)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) ring[d][t] = wl[(d * NT + t) * 64];
+
+#pragma unroll 1
+  for (int ky = 0; ky < 3; ++ky) {
+    int base[3][3];
+#pragma unroll
+    for (int j = 0; j < 3; ++j)
+#pragma unroll
+      for (int kx = 0; kx < 3; ++kx) {
+        const int pp = ci[j] + (ky - 1) * kPitch + (kx - 1);
+        base[j][kx] = pp * G::PIXB + (((h ^ (pp >> 2)) & 1) << 4);
+      }
+    const v4i *wn = wl + (size_t)(ky * U + D) * NT * 64;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int kx = u / KC, kc = u % KC;
+      v4i b[3];
+#pragma unroll
+      for (int j = 0; j < 3; ++j) b[j] = *reinterpret_cast<const v4i *>(smem + base[j][kx] + kc * 32);
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int j = 0; j < 3; ++j) mma<P>(ring[u % D][t], b[j], acc[t][j]);
+      if constexpr (P::SPLIT) {
+        v4i bl[3];
+#pragma unroll
+        for (int j = 0; j < 3; ++j)
+          bl[j] = *reinterpret_cast<const v4i *>(smem + base[j][kx] + kc * 32 + G::PLANE);
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+          for (int j = 0; j < 3; ++j) mma<P>(ring[u % D][t], bl[j], acc[t][j]);
+      }
+#pragma unroll
+      for (int t = 0; t < NT; ++t) ring[u % D][t] = wn[(u * NT + t) * 64];
+    }
+  }
+}
+
+// bias + SiLU + store of one layer's accumulators into the activation tile
+template <class P, int COUT>
+__device__ __forceinline__ void store_activations(unsigned char *smem,
+                                                  const float *__restrict__ bias,
+                                                  const int (&ci)[3], const bool (&valid)[3],
+                                                  int h, const f32x16 (&acc)[COUT / 32][3]) {
+  using G = Geo<P>;
+  constexpr int NT = COUT / 32;
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int ch0 = 32 * t + 8 * q + 4 * h;
+      const f32x4 b4 = *reinterpret_cast<const f32x4 *>(bias + ch0);
+#pragma unroll
+      for (int j = 0; j < 3; ++j) {
+        if (valid[j]) {
+          float v[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = silu<P>(acc[t][j][4 * q + e] + b4[e]);
+          const int off = ci[j] * G::PIXB + ((ch0 * G::EB) ^ (((ci[j] >> 2) & 1) << 4));
+          store4<P>(smem + off, v);
+        }
+      }
+    }
+}
+
+template <int N> __device__ __forceinline__ void zero_acc(f32x16 (&acc)[N][3]) {
+#pragma unroll
+  for (int t = 0; t < N; ++t)
+#pragma unroll
+    for (int j = 0; j < 3; ++j)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[t][j][i] = 0.0f;
+}
+
+template <class P, int L, int CIN, int COUT>
+__device__ __forceinline__ void mid_layer(unsigned char *smem, const unsigned char *packed,
+                                          const float *tail, const int (&ci)[3],
+                                          const bool (&valid)[3], int h, int lane) {
+  using G = Geo<P>;
+  f32x16 acc[COUT / 32][3];
+  zero_acc(acc);
+  const v4i *wl = reinterpret_cast<const v4i *>(packed + (size_t)G::frag_offset(L) * 1024) + lane;
+  conv3_accumulate<P, CIN, COUT>(smem, wl, ci, h, acc);
+  __syncthreads();  // every wave has finished reading the previous layer
+  store_activations<P, COUT>(smem, tail + bias_offset(L), ci, valid, h, acc);
+  __syncthreads();
+}
+
+// ------------------------------------------------------------------------
+// the fused kernel
+// ------------------------------------------------------------------------
+template <class P>
+__global__ __launch_bounds__(kThreads) void fused_forward_kernel(const FwdParams prm) {
+  using G = Geo<P>;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int h = lane >> 5;
+  const int n = lane & 31;
+
+  // per-lane pixel geometry of the three 32-pixel tiles this wave owns
+  int ci[3], l1base[3], pix[3];
+  bool valid[3];
+#pragma unroll
+  for (int j = 0; j < 3; ++j) {
+    const int p = wave * kPixPerWave + j * 32 + n;
+    valid[j] = p < kPix;
+    const int pc = valid[j] ? p : (kPix - 1);
+    pix[j] = pc;
+    const int r = pc / kBoard, c = pc - r * kBoard;
+    ci[j] = (r + 1) * kPitch + (c + 1);
+    const int s = c % G::E;
+    l1base[j] = s * G::COPY_BYTES + ((r * 3 + kL1RowsHalf * h) * kL1RowPitch + (c - s)) * G::EB;
+  }
+
+  unsigned char *occ = smem + G::OCC_OFF;
+  float *lgt = reinterpret_cast<float *>(smem + G::LGT_OFF);
+  float *red = reinterpret_cast<float *>(smem + G::RED_OFF);
+
+  for (long long b = blockIdx.x; b < prm.total_boards; b += gridDim.x) {
+    const long long g = b / prm.boards_per_group;
+    const unsigned char *packed = prm.packed + (size_t)g * prm.packed_stride;
+    const float *tail = reinterpret_cast<const float *>(packed + G::TAIL_OFF);
+
+    __syncthreads();  // previous board fully written out; LDS is free
+    // ---- stage the input: zero the shifted copies, then scatter the board ----
+    {
+      const v4i z = {0, 0, 0, 0};
+      for (int i = tid * 16; i < G::COPIES_BYTES; i += kThreads * 16)
+        *reinterpret_cast<v4i *>(smem + i) = z;
+    }
+    __syncthreads();
+    for (int p = tid; p < kPix; p += kThreads) {
+      const int r = p / kBoard, c = p - r * kBoard;
+      float v[3];
+#pragma unroll
+      for (int ch = 0; ch < 3; ++ch) v[ch] = load_x(prm.x, prm.x_dtype, ((size_t)b * 3 + ch) * kPix + p);
+      unsigned char o = (v[0] != 0.0f) || (v[1] != 0.0f);
+      if (prm.mask_mode == C6_MASK_LEGAL) o = prm.legal[(size_t)b * kPix + p] == 0;
+      if (prm.mask_mode == C6_MASK_NONE) o = 0;
+      occ[p] = o;
+#pragma unroll
+      for (int ch = 0; ch < 3; ++ch) {
+        const int row = (r + kK1 / 2) * 3 + ch;
+#pragma unroll
+        for (int s = 0; s < G::E; ++s) {
+          const int a = s * G::COPY_BYTES + (row * kL1RowPitch + (c + kK1 / 2 - s)) * G::EB;
+          if constexpr (G::EB == 4) {
+            *reinterpret_cast<float *>(smem + a) = v[ch];
+          } else {
+            *reinterpret_cast<unsigned short *>(smem + a) = bits16<P>(v[ch]);
+          }
+        }
+      }
+    }
+    __syncthreads();
+
+    // ---- layer 1 ----
+    {
+      f32x16 acc[1][3];
+      zero_acc(acc);
+      const v4i *wl = reinterpret_cast<const v4i *>(packed) + lane;
+      conv1_accumulate<P>(smem, wl, l1base, acc);
+      __syncthreads();
+      // the copies overlapped the activation tile: restore its zero padding
+      for (int i = tid; i < 60 * (G::PIXB / 16); i += kThreads) {
+        const int k = i / (G::PIXB / 16), w16 = i - k * (G::PIXB / 16);
+        // pad positions: 0..19 (top row), 400..420 (bottom row + tail), 20*R (left column)
+        const int pos = k < 20 ? k : (k < 41 ? 400 + (k - 20) : (k - 40) * kPitch);
+        const v4i z = {0, 0, 0, 0};
+        *reinterpret_cast<v4i *>(smem + pos * G::PIXB + w16 * 16) = z;
+      }
+      store_activations<P, 32>(smem, tail + bias_offset(0), ci, valid, h, acc);
+      __syncthreads();
+    }
+    mid_layer<P, 1, 32, 32>(smem, packed, tail, ci, valid, h, lane);
+    mid_layer<P, 2, 32, 64>(smem, packed, tail, ci, valid, h, lane);
+    mid_layer<P, 3, 64, 64>(smem, packed, tail, ci, valid, h, lane);
+    mid_layer<P, 4, 64, 64>(smem, packed, tail, ci, valid, h, lane);
+    mid_layer<P, 5, 64, 96>(smem, packed, tail, ci, valid, h, lane);
+    mid_layer<P, 6, 96, 96>(smem, packed, tail, ci, valid, h, lane);
+
+    // ---- layer 8 + both 1x1 heads straight from the fp32 accumulators ----
+    {
+      f32x16 acc[3][3];
+      zero_acc(acc);
+      const v4i *wl = reinterpret_cast<const v4i *>(packed + (size_t)G::frag_offset(7) * 1024) + lane;
+      conv3_accumulate<P, 96, 96>(smem, wl, ci, h, acc);
+      const float *bias = tail + bias_offset(7);
+      const float *polw = tail + kBiasTotal;
+      const float *valw = polw + kHeadC;
+      float pol[3] = {0.0f, 0.0f, 0.0f};
+      float vsum = 0.0f;
+#pragma unroll
+      for (int t = 0; t < 3; ++t)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int ch0 = 32 * t + 8 * q + 4 * h;
+          const f32x4 b4 = *reinterpret_cast<const f32x4 *>(bias + ch0);
+          const f32x4 pw = *reinterpret_cast<const f32x4 *>(polw + ch0);
+          const f32x4 vw = *reinterpret_cast<const f32x4 *>(valw + ch0);
+#pragma unroll
+          for (int j = 0; j < 3; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const float a = silu<P>(acc[t][j][4 * q + e] + b4[e]);
+              pol[j] = fmaf(a, pw[e], pol[j]);
+              const float va = a * vw[e];
+              vsum += valid[j] ? va : 0.0f;
+            }
+        }
+      const float polb = valw[kHeadC], valb = valw[kHeadC + 1];
+#pragma unroll
+      for (int j = 0; j < 3; ++j) {
+        const float tot = pol[j] + __shfl_xor(pol[j], 32, 64);
+        if (h == 0 && valid[j]) lgt[pix[j]] = tot + polb;
+      }
+      vsum = wave_sum(vsum);
+      if (lane == 0) red[wave] = vsum;
+      __syncthreads();
+      if (tid == 0 && prm.value != nullptr) {
+        const float s = (red[0] + red[1]) + (red[2] + red[3]);
+        prm.value[b] = tanhf(s * (1.0f / kPix) + valb);
+      }
+    }
+
+    // ---- write out: masked logits, optional sampled action ----
+    if (prm.logits != nullptr) {
+      for (int p = tid; p < kPix; p += kThreads) {
+        const float v = lgt[p];
+        prm.logits[(size_t)b * kPix + p] = occ[p] ? prm.fill : v;
+      }
+    }
+    if (prm.actions != nullptr && wave == 0) {
+      const float it = prm.inv_temperature;
+      int a;
+      float lp;
+      wave_sample(
+          lane, prm.u[b], [&](int i) { return lgt[i] * it; }, [&](int i) { return occ[i] == 0; },
+          a, lp);
+      if (lane == 0) {
+        prm.actions[b] = a;
+        if (prm.logprob != nullptr) prm.logprob[b] = lp;
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------
+// weight repack: PyTorch OIHW fp32 -> MFMA fragment order
+// ------------------------------------------------------------------------
+template <class P> __device__ __forceinline__ void put_elem(unsigned char *dst, int e, float v) {
+  if constexpr (P::EB == 4) {
+    reinterpret_cast<float *>(dst)[e] = v;
+  } else {
+    reinterpret_cast<unsigned short *>(dst)[e] = bits16<P>(v);
+  }
+}
+
+// one thread per (fragment, lane): writes the 16 bytes that lane will load
+template <class P> __global__ void pack_kernel(const PackParams prm) {
+  using G = Geo<P>;
+  const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long long nfl = (long long)G::TOTAL_FRAGS * 64;
+  if (gid < nfl) {
+    const int frag = (int)(gid >> 6), lane = (int)(gid & 63);
+    const int m = lane & 31, h = lane >> 5;
+    unsigned char *dst = prm.packed + (size_t)gid * 16;
+    int l = 0;
+    while (l < 8 && frag >= G::frag_offset(l + 1)) ++l;  // frag_offset is monotone
+    if (l >= 8) {  // over-read padding
+      *reinterpret_cast<v4i *>(dst) = v4i{0, 0, 0, 0};
+      return;
+    }
+    const int fi = frag - G::frag_offset(l);
+    const int cin = kCinArr[l], cout = kCoutArr[l];
+    const int nt = cout / 32;
+    const int s = fi / nt, t = fi - s * nt;
+    const int co = 32 * t + m;
+    const float *w = prm.conv_w[l];
+    if (l == 0) {
+      const int row = s / G::CPR + kL1RowsHalf * h;  // (ky, plane) row, 69 real + 1 pad
+      const int jj = s % G::CPR;
+      const int ky = row / 3, ch = row - ky * 3;
+      for (int e = 0; e < G::E; ++e) {
+        const int kx = jj * G::E + e;
+        float v = 0.0f;
+        if (row < kK1 * 3 && kx < kK1) v = w[((co * 3 + ch) * kK1 + ky) * kK1 + kx];
+        put_elem<P>(dst, e, v);
+      }
+    } else {
+      const int kc_per_tap = cin / G::KSTEP;
+      const int tap = s / kc_per_tap, kc = s - tap * kc_per_tap;
+      for (int e = 0; e < G::E; ++e) {
+        const int c = kc * G::KSTEP + h * G::E + e;
+        put_elem<P>(dst, e, w[(co * cin + c) * 9 + tap]);
+      }
+    }
+    return;
+  }
+  // fp32 tail: biases, head weights, head biases
+  const int ti = (int)(gid - nfl);
+  if (ti < G::TAIL_FLOATS) {
+    float *tail = reinterpret_cast<float *>(prm.packed + G::TAIL_OFF);
+    float v = 0.0f;
+    if (ti < kBiasTotal) {
+      int l = 0;
+      while (ti >= bias_offset(l + 1)) ++l;
+      v = prm.conv_b[l] ? prm.conv_b[l][ti - bias_offset(l)] : 0.0f;
+    } else if (ti < kBiasTotal + kHeadC) {
+      v = prm.pol_w[ti - kBiasTotal];
+    } else if (ti < kBiasTotal + 2 * kHeadC) {
+      v = prm.val_w ? prm.val_w[ti - kBiasTotal - kHeadC] : 0.0f;
+    } else if (ti == kBiasTotal + 2 * kHeadC) {
+      v = prm.pol_b ? prm.pol_b[0] : 0.0f;
+    } else if (ti == kBiasTotal + 2 * kHeadC + 1) {
+      v = prm.val_b ? prm.val_b[0] : 0.0f;
+    }
+    tail[ti] = v;
+  }
+}
+
+// ------------------------------------------------------------------------
+// host side
+// ------------------------------------------------------------------------
+template <class P> static int launch_pack(const PackParams &pp, hipStream_t st) {
+  using G = Geo<P>;
+  const long long total = (long long)G::TOTAL_FRAGS * 64 + G::TAIL_FLOATS;
+  const int threads = 256;
+  const int blocks = (int)((total + threads - 1) / threads);
+  hipLaunchKernelGGL(pack_kernel<P>, dim3(blocks), dim3(threads), 0, st, pp);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    set_error("pack_kernel launch failed: %s", hipGetErrorString(e));
+    return C6_ELAUNCH;
+  }
+  return C6_OK;
+}
+
+template <class P> static int launch_forward(const FwdParams &fp, hipStream_t st) {
+  using G = Geo<P>;
+  static_assert(G::LDS_BYTES <= 160 * 1024, "activation tile must fit the 160 KiB LDS of a CU");
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  static thread_local int configured_dev[4] = {-1, -1, -1, -1};
+  static thread_local int cus[4] = {0, 0, 0, 0};
+  if (e == hipSuccess && configured_dev[P::ID] != dev) {
+    e = hipFuncSetAttribute(reinterpret_cast<const void *>(&fused_forward_kernel<P>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, G::LDS_BYTES);
+    int n = 0;
+    if (e == hipSuccess) e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e == hipSuccess) {
+      configured_dev[P::ID] = dev;
+      cus[P::ID] = n;
+    }
+  }
+  if (e != hipSuccess) {
+    set_error("fused_forward setup failed: %s", hipGetErrorString(e));
+    return C6_ELAUNCH;
+  }
+  long long grid = cus[P::ID] > 0 ? cus[P::ID] : 256;
+  if (grid > fp.total_boards) grid = fp.total_boards;
+  hipLaunchKernelGGL(fused_forward_kernel<P>, dim3((unsigned)grid), dim3(kThreads), G::LDS_BYTES,
+                     st, fp);
+  e = hipGetLastError();
+  if (e != hipSuccess) {
+    set_error("fused_forward launch failed: %s", hipGetErrorString(e));
+    return C6_ELAUNCH;
+  }
+  return C6_OK;
+}
+
+int dispatch_pack(int prec, const PackParams &pp, hipStream_t st) {
+  switch (prec) {
+    case C6_PREC_F32: return launch_pack<PrecF32>(pp, st);
+    case C6_PREC_BF16: return launch_pack<PrecBF16>(pp, st);
+    case C6_PREC_F16: return launch_pack<PrecF16>(pp, st);
+    case C6_PREC_BF16X2: return launch_pack<PrecBF16X2>(pp, st);
+  }
+  set_error("unknown precision mode %d", prec);
+  return C6_EINVAL;
+}
+
+int dispatch_forward(int prec, const FwdParams &fp, hipStream_t st) {
+  switch (prec) {
+    case C6_PREC_F32: return launch_forward<PrecF32>(fp, st);
+    case C6_PREC_BF16: return launch_forward<PrecBF16>(fp, st);
+    case C6_PREC_F16: return launch_forward<PrecF16>(fp, st);
+    case C6_PREC_BF16X2: return launch_forward<PrecBF16X2>(fp, st);
+  }
+  set_error("unknown precision mode %d", prec);
+  return C6_EINVAL;
+}
+
+size_t packed_bytes(int prec) {
+  switch (prec) {
+    case C6_PREC_F32: return Geo<PrecF32>::PACKED_BYTES;
+    case C6_PREC_BF16: return Geo<PrecBF16>::PACKED_BYTES;
+    case C6_PREC_F16: return Geo<PrecF16>::PACKED_BYTES;
+    case C6_PREC_BF16X2: return Geo<PrecBF16X2>::PACKED_BYTES;
+  }
+  return 0;
+}
+
+}  // namespace c6

@@ -1,0 +1,349 @@
+"""Drop-in ``PolicyValueNet`` whose forward runs hand-written HIP kernels.
+
+Mirrors the operator interface of the reference's connect6/model.py
+(``PolicyValueNet``, ``build_model``, ``mask_logits``): same constructor,
+validation, attributes, ``state_dict`` keys and error behaviour.  The forward
+pass itself is one fused gfx950 kernel launched through the C ABI in
+``include/connect6_amd.h``; PyTorch only owns the memory and the stream.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Any
+
+import torch
+from torch import nn
+
+from . import _lib
+
+_FILL_LOWEST = float(torch.finfo(torch.float32).min)
+
+
+def _require_device_tensor(t: torch.Tensor, what: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(
+            f"{what} is on {t.device}: connect6_amd computes only on an MI355X (HIP) device; "
+            "there is no CPU path"
+        )
+
+
+def pack_state(state: dict[str, torch.Tensor], prec: int, out: torch.Tensor) -> None:
+    """Repack one checkpoint (reference ``state_dict`` keys, device tensors)
+    into ``out`` (uint8 device buffer of ``_lib.packed_bytes(prec)`` bytes)."""
+    lib = _lib.load()
+    keep = []  # keep fp32 staging copies alive until the launch is enqueued
+
+    def dev32(key: str, required: bool = True):
+        if key not in state:
+            if required:
+                raise KeyError(f"missing parameter {key}")
+            return None
+        t = state[key].detach().to(device=out.device, dtype=torch.float32).contiguous()
+        keep.append(t)
+        return t
+
+    ws = [dev32(f"convs.{i}.weight") for i in range(8)]
+    bs = [dev32(f"convs.{i}.bias", required=False) for i in range(8)]
+    expect_in = 3
+    for i, (k, c) in enumerate(zip(PolicyValueNet.DEFAULT_KERNELS, PolicyValueNet.DEFAULT_CHANNELS)):
+        if tuple(ws[i].shape) != (c, expect_in, k, k):
+            raise ValueError(
+                f"convs.{i}.weight has shape {tuple(ws[i].shape)}; the fused kernels are built for "
+                f"the default architecture and need {(c, expect_in, k, k)}"
+            )
+        expect_in = c
+    pw, pb = dev32("policy_output.weight"), dev32("policy_output.bias", required=False)
+    vw, vb = dev32("value_output.weight", required=False), dev32("value_output.bias", required=False)
+    vp = ctypes.c_void_p
+    wptrs = (vp * 8)(*[t.data_ptr() for t in ws])
+    bptrs = (vp * 8)(*[(t.data_ptr() if t is not None else None) for t in bs])
+
+    def ptr(t):
+        return t.data_ptr() if t is not None else None
+
+    with torch.cuda.device(out.device):
+        rc = lib.c6_pack_weights(wptrs, bptrs, ptr(pw), ptr(pb), ptr(vw), ptr(vb), prec,
+                                 out.data_ptr(), _lib.stream_ptr(out.device))
+    _lib.check(rc, "c6_pack_weights")
+    # the staging copies are freed by the caching allocator in stream order, after the kernel
+
+
+def run_forward(
+    x: torch.Tensor,
+    packed: torch.Tensor,
+    prec: int,
+    groups: int,
+    boards_per_group: int,
+    *,
+    want_logits: bool = True,
+    want_value: bool = True,
+    mask_mode: int = _lib.MASK_NONE,
+    legal: torch.Tensor | None = None,
+    fill: float = _FILL_LOWEST,
+    u: torch.Tensor | None = None,
+    temperature: float = 1.0,
+    want_logprob: bool = False,
+):
+    """Launch ``c6_forward``; returns (logits, value, actions, logprob), each
+    None when not requested."""
+    lib = _lib.load()
+    dev = x.device
+    total = groups * boards_per_group
+    x = x.contiguous()
+    logits = torch.empty((total, 361), dtype=torch.float32, device=dev) if want_logits else None
+    value = torch.empty((total,), dtype=torch.float32, device=dev) if want_value else None
+    actions = logprob = None
+    if u is not None:
+        u = u.to(device=dev, dtype=torch.float32).contiguous()
+        if u.shape != (total,):
+            raise ValueError(f"u must have shape ({total},), got {tuple(u.shape)}")
+        actions = torch.empty((total,), dtype=torch.int64, device=dev)
+        if want_logprob:
+            logprob = torch.empty((total,), dtype=torch.float32, device=dev)
+    if legal is not None:
+        if legal.shape != (total, 361):
+            raise ValueError(f"legal mask must have shape ({total}, 361), got {tuple(legal.shape)}")
+        if legal.dtype == torch.bool:
+            legal = legal.contiguous().view(torch.uint8)
+        elif legal.dtype != torch.uint8:
+            raise ValueError("legal mask must be a bool or uint8 tensor")
+        legal = legal.to(dev).contiguous()
+
+    def ptr(t):
+        return t.data_ptr() if t is not None else None
+
+    stride = packed.numel() // groups if groups > 1 else packed.numel()
+    with torch.cuda.device(dev):
+        rc = lib.c6_forward(x.data_ptr(), _lib.torch_dtype_code(x.dtype), groups, boards_per_group,
+                            packed.data_ptr(), stride, prec, ptr(logits), ptr(value), mask_mode,
+                            ptr(legal), fill, ptr(u), float(temperature), ptr(actions),
+                            ptr(logprob), _lib.stream_ptr(dev))
+    _lib.check(rc, "c6_forward")
+    return logits, value, actions, logprob
+
+
+class PolicyValueNet(nn.Module):
+    """Fully convolutional policy + value network for Connect6
+    (reference: connect6/model.py:9-111).
+
+    Input ``[B, 3, H, W]``: 0 = own stones, 1 = opponent stones, 2 = whether
+    this decision is the last stone of the turn.  Returns ``(logits[B, H*W],
+    value[B])``, both fp32.
+
+    ``precision`` selects the arithmetic of the HIP path: ``None`` follows
+    PyTorch's own rules (bf16/fp16 under ``torch.autocast`` or when the
+    parameters are held in that dtype, else fp32); or one of ``"fp32"``,
+    ``"bf16"``, ``"fp16"``, ``"bf16x2"`` (bf16 MFMA with activations carried
+    as a hi+lo bf16 pair).
+    """
+
+    DEFAULT_KERNELS = (23, 3, 3, 3, 3, 3, 3, 3)
+    DEFAULT_CHANNELS = (32, 32, 64, 64, 64, 96, 96, 96)
+    INPUT_CHANNELS = 3
+
+    def __init__(
+        self,
+        board_size: int = 19,
+        kernels: list[int] | tuple[int, ...] | None = None,
+        channels: list[int] | tuple[int, ...] | None = None,
+    ) -> None:
+        super().__init__()
+        self.board_size = int(board_size)
+        self.action_size = self.board_size * self.board_size
+        self.input_channels = self.INPUT_CHANNELS
+
+        kernels = tuple(self.DEFAULT_KERNELS if kernels is None else kernels)
+        channels = tuple(self.DEFAULT_CHANNELS if channels is None else channels)
+        # same checks, same order, same exception type as connect6/model.py:40-47
+        if len(kernels) != len(channels):
+            raise ValueError("kernels and channels must have the same number of elements")
+        if not kernels:
+            raise ValueError("the CNN needs at least one layer")
+        if any(k <= 0 or k % 2 == 0 for k in kernels):
+            raise ValueError("every kernel must be a positive odd number")
+        if any(c <= 0 for c in channels):
+            raise ValueError("channel counts must be positive")
+        self.kernels = kernels
+        self.channels = channels
+
+        convs = []
+        cin = self.input_channels
+        for k, cout in zip(kernels, channels):
+            convs.append(nn.Conv2d(cin, cout, kernel_size=k, stride=1, padding=k // 2, bias=True))
+            cin = cout
+        self.convs = nn.ModuleList(convs)
+        self.activation = nn.SiLU(inplace=True)
+        self.policy_output = nn.Conv2d(cin, 1, kernel_size=1, bias=True)
+        self.value_output = nn.Conv2d(cin, 1, kernel_size=1, bias=True)
+        self.value_tanh = nn.Tanh()
+        self._init_weights()
+
+        self.precision: str | None = None
+        self._packed: dict[int, tuple[tuple, torch.Tensor]] = {}
+
+    @property
+    def receptive_field(self) -> int:
+        return 1 + sum(k - 1 for k in self.kernels)
+
+    def _init_weights(self) -> None:
+        """connect6/model.py:83-94: Kaiming-normal (ReLU gain) convs with zero
+        bias; both heads N(0, 0.01) with zero bias."""
+        for conv in self.convs:
+            nn.init.kaiming_normal_(conv.weight, nonlinearity="relu")
+            if conv.bias is not None:
+                nn.init.zeros_(conv.bias)
+        for head in (self.policy_output, self.value_output):
+            nn.init.normal_(head.weight, mean=0.0, std=0.01)
+            nn.init.zeros_(head.bias)
+
+    # -- precision / weights ------------------------------------------------
+    @property
+    def is_default_architecture(self) -> bool:
+        return (
+            self.board_size == 19
+            and self.kernels == self.DEFAULT_KERNELS
+            and self.channels == self.DEFAULT_CHANNELS
+        )
+
+    def resolve_precision(self) -> int:
+        if self.precision is not None:
+            try:
+                return _lib.PREC_BY_NAME[self.precision]
+            except KeyError:
+                raise ValueError(
+                    f"precision must be one of {sorted(_lib.PREC_BY_NAME)} or None, got {self.precision!r}"
+                ) from None
+        dtype = self.convs[0].weight.dtype
+        if torch.is_autocast_enabled():  # reference: train.py:126-130 wraps calls in autocast
+            dtype = torch.get_autocast_gpu_dtype()
+        if dtype == torch.bfloat16:
+            return _lib.PREC_BF16
+        if dtype == torch.float16:
+            return _lib.PREC_F16
+        return _lib.PREC_F32
+
+    def packed_weights(self, prec: int) -> torch.Tensor:
+        """Kernel-layout copy of the parameters; rebuilt whenever a parameter
+        was modified in place, replaced or moved."""
+        params = list(self.parameters())
+        key = tuple((p.data_ptr(), p._version, p.dtype) for p in params)
+        hit = self._packed.get(prec)
+        if hit is not None and hit[0] == key:
+            return hit[1]
+        dev = params[0].device
+        buf = torch.empty(_lib.packed_bytes(prec), dtype=torch.uint8, device=dev)
+        pack_state({k: v for k, v in self.state_dict().items()}, prec, buf)
+        self._packed[prec] = (key, buf)
+        return buf
+
+    # -- forward --------------------------------------------------------------
+    def _check_input(self, x: torch.Tensor) -> None:
+        expected = (self.input_channels, self.board_size, self.board_size)
+        if x.ndim != 4 or tuple(x.shape[1:]) != expected:
+            raise ValueError(
+                f"model input must have shape [B, {expected[0]}, {expected[1]}, {expected[2]}], "
+                f"got {tuple(x.shape)}."
+            )
+        _require_device_tensor(x, "model input")
+        _require_device_tensor(self.convs[0].weight, "model parameters")
+        if torch.is_grad_enabled() and (
+            x.requires_grad or any(p.requires_grad for p in self.parameters())
+        ):
+            raise RuntimeError(
+                "connect6_amd.PolicyValueNet is the inference forward only: call it under "
+                "torch.no_grad() / torch.inference_mode() (training stays on a PyTorch module "
+                "sharing this state_dict)"
+            )
+        if not self.is_default_architecture:
+            raise NotImplementedError(
+                "the HIP kernels are built for board 19, kernels "
+                f"{self.DEFAULT_KERNELS}, channels {self.DEFAULT_CHANNELS}; got board "
+                f"{self.board_size}, kernels {self.kernels}, channels {self.channels}"
+            )
+
+    def forward(self, x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+        self._check_input(x)
+        prec = self.resolve_precision()
+        logits, value, _, _ = run_forward(x, self.packed_weights(prec), prec, 1, int(x.shape[0]))
+        return logits, value
+
+    def forward_masked(
+        self,
+        x: torch.Tensor,
+        legal: torch.Tensor | None = None,
+        fill: float | None = None,
+    ) -> tuple[torch.Tensor, torch.Tensor]:
+        """Forward with the occupied-square masking fused into the head:
+        equals ``mask_logits(forward(x)[0].float(), legal)``.  With
+        ``legal=None`` a square is occupied iff plane 0 or plane 1 of ``x`` is
+        non-zero there.  ``fill`` defaults to ``finfo(float32).min``."""
+        self._check_input(x)
+        prec = self.resolve_precision()
+        logits, value, _, _ = run_forward(
+            x, self.packed_weights(prec), prec, 1, int(x.shape[0]),
+            mask_mode=_lib.MASK_INPUT if legal is None else _lib.MASK_LEGAL, legal=legal,
+            fill=_FILL_LOWEST if fill is None else float(fill),
+        )
+        return logits, value
+
+    def selfplay_step(
+        self,
+        x: torch.Tensor,
+        u: torch.Tensor,
+        temperature: float = 1.0,
+        legal: torch.Tensor | None = None,
+        return_logits: bool = False,
+    ):
+        """Fused collector step: forward, occupied-square mask, masked softmax
+        at ``temperature`` and one categorical draw per board by inverse CDF
+        on ``u[b]`` in [0,1) -- the work of ``_sample_actions`` in the
+        reference (connect6/train.py:195-203) without materialising logits.
+        Returns ``(actions int64[B], logprob[B], value[B])`` (+ masked logits)."""
+        self._check_input(x)
+        prec = self.resolve_precision()
+        logits, value, actions, logprob = run_forward(
+            x, self.packed_weights(prec), prec, 1, int(x.shape[0]), want_logits=return_logits,
+            mask_mode=_lib.MASK_INPUT if legal is None else _lib.MASK_LEGAL, legal=legal,
+            u=u, temperature=temperature, want_logprob=True,
+        )
+        if return_logits:
+            return actions, logprob, value, logits
+        return actions, logprob, value
+
+
+def build_model(model_cfg: dict[str, Any], board_size: int) -> PolicyValueNet:
+    """Build the CNN from the ``model`` section of the YAML config
+    (connect6/model.py:114-120): the three bookkeeping keys are ignored."""
+    cfg = dict(model_cfg)
+    cfg.pop("compile", None)
+    cfg.pop("compile_mode", None)
+    cfg.pop("architecture_version", None)
+    return PolicyValueNet(board_size=board_size, **cfg)
+
+
+def mask_logits(logits: torch.Tensor, legal_mask: torch.Tensor) -> torch.Tensor:
+    """Block occupied squares so that a softmax can never choose them
+    (connect6/model.py:123-125): out-of-place, fill = ``finfo(dtype).min``."""
+    _require_device_tensor(logits, "logits")
+    if logits.ndim != 2 or logits.shape[1] != 361 or legal_mask.shape != logits.shape:
+        raise ValueError(
+            f"mask_logits expects logits and legal mask of shape [B, 361], got "
+            f"{tuple(logits.shape)} and {tuple(legal_mask.shape)}"
+        )
+    if legal_mask.dtype != torch.bool:
+        raise ValueError("legal mask must be a bool tensor")
+    lib = _lib.load()
+    src = logits.contiguous()
+    legal = legal_mask.to(logits.device).contiguous().view(torch.uint8)
+    out = torch.empty_like(src)
+    fill = torch.tensor(torch.finfo(src.dtype).min, dtype=src.dtype)
+    if src.dtype == torch.float32:
+        fill_bits = int(fill.view(torch.int32).item()) & 0xFFFFFFFF
+    else:
+        fill_bits = int(fill.view(torch.int16).item()) & 0xFFFF
+    with torch.cuda.device(src.device):
+        rc = lib.c6_mask_logits(src.data_ptr(), legal.data_ptr(), _lib.torch_dtype_code(src.dtype),
+                                int(src.shape[0]), fill_bits, out.data_ptr(),
+                                _lib.stream_ptr(src.device))
+    _lib.check(rc, "c6_mask_logits")
+    return out

@@ -1,0 +1,121 @@
+/* connect6_amd -- C ABI of the MI355X (gfx950) Connect6 policy/value forward path.
+ *
+ * One shared library, plain pointers and sizes only.  Every pointer named
+ * "device" is a HIP device pointer owned by the caller (PyTorch in the shipped
+ * host code); the library never allocates, frees or keeps device memory, and
+ * every call only enqueues work on the caller's stream (no synchronisation).
+ * All functions return C6_OK (0) or a negative C6_E* code; c6_last_error()
+ * gives the message of the calling thread's last failure.
+ *
+ * The reference implementation is pure Python on PyTorch, so it has no FFI of
+ * its own; each entry point below names the reference call it replaces.
+ */
+#ifndef CONNECT6_AMD_H
+#define CONNECT6_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define C6_BOARD 19
+#define C6_ACTIONS 361
+#define C6_LAYERS 8
+
+/* return codes */
+#define C6_OK 0
+#define C6_EINVAL (-1)   /* bad shape / dtype / null pointer / alignment */
+#define C6_ELAUNCH (-2)  /* HIP reported an error at launch */
+#define C6_EARCH (-3)    /* device is not gfx950 or architecture not the default one */
+
+/* arithmetic modes of the network ("prec") */
+#define C6_PREC_F32 0    /* fp32 operands, fp32 MFMA                                        */
+#define C6_PREC_BF16 1   /* bf16 operands, bf16 MFMA, fp32 accumulate, bf16 layer boundaries */
+#define C6_PREC_F16 2    /* fp16 operands, fp16 MFMA, fp32 accumulate, fp16 layer boundaries */
+#define C6_PREC_BF16X2 3 /* bf16 MFMA, activations carried as a bf16 hi+lo pair (two passes)  */
+
+/* element types of caller tensors */
+#define C6_DT_F32 0
+#define C6_DT_BF16 1
+#define C6_DT_F16 2
+
+/* masking of occupied squares in the policy logits */
+#define C6_MASK_NONE 0   /* logits as the network produced them (PolicyValueNet.forward)    */
+#define C6_MASK_INPUT 1  /* square occupied iff x[b,0,r,c] != 0 or x[b,1,r,c] != 0           */
+#define C6_MASK_LEGAL 2  /* square occupied iff legal[b,a] == 0 (uint8 / torch.bool tensor)  */
+
+int c6_version(void);
+const char *c6_last_error(void);
+
+/* Size in bytes of one packed weight set for arithmetic mode `prec`. */
+int c6_packed_bytes(int prec, size_t *bytes);
+
+/* Repack one checkpoint's parameters for the kernels.
+ * Replaces: the parameter tensors nn.Conv2d holds in PolicyValueNet.__init__
+ * (connect6/model.py:52-75) and the per-key stacking of
+ * HistoricalPolicyEnsemble._stack (connect6/history.py:224-240).
+ * conv_w[i] / conv_b[i]: device fp32, PyTorch layouts [Cout,Cin,k,k] / [Cout]
+ * for the default architecture (kernels 23,3x7; channels 32,32,64,64,64,96,96,96);
+ * conv_b[i] may be NULL (no bias).  pol_* / val_*: device fp32 [1,96,1,1] / [1];
+ * val_w / val_b may be NULL (history checkpoints need no value head).
+ * `conv_w` and `conv_b` themselves are HOST arrays of 8 device pointers.
+ * `packed`: device buffer of c6_packed_bytes(prec) bytes, 16-byte aligned. */
+int c6_pack_weights(const float *const *conv_w, const float *const *conv_b,
+                    const float *pol_w, const float *pol_b, const float *val_w,
+                    const float *val_b, int prec, void *packed, void *stream);
+
+/* Batched forward of G weight sets, each applied to T boards, in one launch.
+ * Replaces: PolicyValueNet.forward (connect6/model.py:96-111) with G = 1, and
+ * HistoricalPolicyEnsemble.forward_grouped (connect6/history.py:276-303) with
+ * G = number of checkpoints (value == NULL there: policy only).
+ *   x       device [G*T,3,19,19] contiguous, element type x_dtype
+ *   packed  device, G weight sets, consecutive sets `packed_stride` bytes apart
+ *   logits  device fp32 [G*T,361] (may be NULL)
+ *   value   device fp32 [G*T] (may be NULL)
+ *   mask_mode / legal / fill: see C6_MASK_*; `fill` is stored bit-exactly in
+ *           every masked logit (connect6/model.py:123-125 uses finfo.min).
+ * Optional fused sampling (connect6/train.py:195-213, _sample_actions): when
+ * `actions` is not NULL, each board also draws an action by inverse CDF on
+ * u[b] in [0,1) from softmax(masked_logits / max(temperature,1e-4)) (masking
+ * as selected by mask_mode, always with fill = lowest float) and writes
+ * actions[b] (int64) and, if not NULL, logprob[b] (fp32). */
+int c6_forward(const void *x, int x_dtype, int64_t groups, int64_t boards_per_group,
+               const void *packed, size_t packed_stride, int prec, float *logits,
+               float *value, int mask_mode, const uint8_t *legal, float fill,
+               const float *u, float temperature, int64_t *actions, float *logprob,
+               void *stream);
+
+/* Out-of-place occupied-square masking of existing logits.
+ * Replaces: mask_logits (connect6/model.py:123-125).
+ * logits/out: device [B,361] of element type dtype; legal: device uint8 [B,361];
+ * fill_bits: the fill value's bit pattern in that element type. */
+int c6_mask_logits(const void *logits, const uint8_t *legal, int dtype, int64_t batch,
+                   uint32_t fill_bits, void *out, void *stream);
+
+/* Masked softmax + inverse-CDF categorical sampling of existing logits.
+ * Replaces: _sample_actions / _sample_actions_only (connect6/train.py:195-213).
+ * logits fp32 [B,361]; legal uint8 [B,361] or NULL; u fp32 [B] in [0,1);
+ * actions int64 [B]; logprob fp32 [B] or NULL. */
+int c6_softmax_sample(const float *logits, const uint8_t *legal, const float *u,
+                      float temperature, int64_t batch, int64_t *actions, float *logprob,
+                      void *stream);
+
+/* Eight D4 views of network inputs, in the order of _symmetry_for_phase
+ * (connect6/train.py:216-219); view p is _transform_boards(x, p%4, p>=4)
+ * (connect6/train.py:222-230).  x: device [B,3,19,19]; out: [8,B,3,19,19];
+ * both of element type dtype. */
+int c6_d4_expand(const void *x, int dtype, int64_t batch, void *out, void *stream);
+
+/* Map the eight views' logits back with _transform_actions
+ * (connect6/train.py:233-253) and average logits and values over the views.
+ * view_logits fp32 [8,B,361], view_values fp32 [8,B] (may be NULL with values);
+ * logits fp32 [B,361]; values fp32 [B]. */
+int c6_d4_reduce(const float *view_logits, const float *view_values, int64_t batch,
+                 float *logits, float *values, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CONNECT6_AMD_H */
