@@ -180,6 +180,8 @@ class PolicyValueNet(nn.Module):
 
         self.precision: str | None = None
         self._packed: dict[int, tuple[tuple, torch.Tensor]] = {}
+        self._epoch = 0
+        self.register_load_state_dict_post_hook(lambda module, _keys: module.refresh_weights())
 
     @property
     def receptive_field(self) -> int:
@@ -214,19 +216,28 @@ class PolicyValueNet(nn.Module):
                     f"precision must be one of {sorted(_lib.PREC_BY_NAME)} or None, got {self.precision!r}"
                 ) from None
         dtype = self.convs[0].weight.dtype
-        if torch.is_autocast_enabled():  # reference: train.py:126-130 wraps calls in autocast
-            dtype = torch.get_autocast_gpu_dtype()
+        if torch.is_autocast_enabled("cuda"):  # reference: train.py:126-130 wraps calls in autocast
+            dtype = torch.get_autocast_dtype("cuda")
         if dtype == torch.bfloat16:
             return _lib.PREC_BF16
         if dtype == torch.float16:
             return _lib.PREC_F16
         return _lib.PREC_F32
 
+    def refresh_weights(self) -> None:
+        """Force a repack on the next forward (needed only after modifying
+        parameters that were created under ``torch.inference_mode()`` in place;
+        ordinary in-place updates, ``load_state_dict`` and ``.to()`` are seen)."""
+        self._epoch += 1
+
     def packed_weights(self, prec: int) -> torch.Tensor:
         """Kernel-layout copy of the parameters; rebuilt whenever a parameter
         was modified in place, replaced or moved."""
         params = list(self.parameters())
-        key = tuple((p.data_ptr(), p._version, p.dtype) for p in params)
+        # inference tensors carry no version counter; load_state_dict / refresh_weights bump the epoch
+        key = (self._epoch,) + tuple(
+            (p.data_ptr(), -1 if p.is_inference() else p._version, p.dtype) for p in params
+        )
         hit = self._packed.get(prec)
         if hit is not None and hit[0] == key:
             return hit[1]

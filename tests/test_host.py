@@ -1,0 +1,210 @@
+"""Host-side logic of the drop-in modules and the C-ABI surface, no GPU needed
+(no compute entry point is launched here)."""
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+import torch
+
+import connect6_amd as c6
+from connect6_amd import _lib
+from oracle import torch_ref as R
+
+ROOT = Path(__file__).resolve().parent.parent
+
+
+def test_library_exports_every_declared_symbol():
+    header = (ROOT / "include" / "connect6_amd.h").read_text()
+    declared = set(re.findall(r"\b(c6_[a-z0-9_]+)\s*\(", header))
+    assert declared == set(_lib.EXPORTS)
+    lib = _lib.load()
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert lib.c6_version() == 1
+
+
+def test_packed_sizes_follow_the_layout():
+    # 1 KiB fragments: first layer 35 rows x (24/E) per half, 3x3 layers 9*Cin/KSTEP x Cout/32
+    def frags(e):
+        kstep = 2 * e
+        n = 35 * (24 // e)
+        for cin, cout in zip((32, 32, 64, 64, 64, 96, 96), (32, 64, 64, 64, 96, 96, 96)):
+            n += (9 * cin // kstep) * (cout // 32)
+        return n + 24
+    tail = (544 + 96 + 96 + 4) * 4
+    assert _lib.packed_bytes(_lib.PREC_BF16) == frags(8) * 1024 + tail
+    assert _lib.packed_bytes(_lib.PREC_F16) == frags(8) * 1024 + tail
+    assert _lib.packed_bytes(_lib.PREC_BF16X2) == frags(8) * 1024 + tail
+    assert _lib.packed_bytes(_lib.PREC_F32) == frags(4) * 1024 + tail
+    with pytest.raises(ValueError):
+        _lib.packed_bytes(9)
+
+
+def test_entry_points_reject_bad_arguments_before_touching_the_device():
+    lib = _lib.load()
+    assert lib.c6_forward(None, 0, 1, 4, None, 0, 1, None, None, 0, None, 0.0, None, 1.0, None, None, None) == -1
+    assert b"null" in lib.c6_last_error()
+    assert lib.c6_forward(None, 7, 1, 4, None, 0, 1, None, None, 0, None, 0.0, None, 1.0, None, None, None) == -1
+    assert lib.c6_forward(None, 0, 1, 4, None, 0, 5, None, None, 0, None, 0.0, None, 1.0, None, None, None) == -1
+    assert lib.c6_forward(None, 0, 0, 4, None, 0, 1, None, None, 0, None, 0.0, None, 1.0, None, None, None) == -1
+    # an empty batch is a no-op, not an error
+    assert lib.c6_forward(None, 0, 1, 0, None, 0, 1, None, None, 0, None, 0.0, None, 1.0, None, None, None) == 0
+    assert lib.c6_mask_logits(None, None, 0, 3, 0, None, None) == -1
+    assert lib.c6_mask_logits(None, None, 0, 0, 0, None, None) == 0
+    assert lib.c6_softmax_sample(None, None, None, 1.0, 2, None, None, None) == -1
+    assert lib.c6_d4_expand(None, 0, 2, None, None) == -1
+    assert lib.c6_d4_reduce(None, None, 2, None, None, None) == -1
+    assert lib.c6_pack_weights(None, None, None, None, None, None, 1, None, None) == -1
+
+
+def test_model_attributes_match_reference_contract():
+    # tests/test_model.py:11-37 of the reference, minus the CPU forward
+    model = c6.PolicyValueNet(board_size=19)
+    assert model.receptive_field == 37
+    assert model.board_size == 19 and model.action_size == 361 and model.input_channels == 3
+    cfg = {
+        "architecture_version": 4,
+        "kernels": [23, 3, 3, 3, 3, 3, 3, 3],
+        "channels": [32, 32, 64, 64, 64, 96, 96, 96],
+        "compile": False,
+        "compile_mode": "default",
+    }
+    model = c6.build_model(cfg, 19)
+    assert [m.kernel_size[0] for m in model.convs] == [23, 3, 3, 3, 3, 3, 3, 3]
+    assert [m.out_channels for m in model.convs] == [32, 32, 64, 64, 64, 96, 96, 96]
+    assert model.convs[0].in_channels == 3
+    assert model.policy_output.kernel_size == (1, 1)
+    assert model.policy_output.in_channels == 96
+    assert model.policy_output.out_channels == 1
+    assert model.value_output.kernel_size == (1, 1)
+    assert model.receptive_field == 37
+    assert model.kernels == (23, 3, 3, 3, 3, 3, 3, 3)
+    assert isinstance(model.activation, torch.nn.SiLU)
+
+
+def test_state_dict_is_interchangeable_with_the_oracle():
+    model = c6.PolicyValueNet()
+    st = R.init_state(1, "reference")
+    assert set(model.state_dict().keys()) == set(st.keys())
+    for k, v in model.state_dict().items():
+        assert v.shape == st[k].shape, k
+    model.load_state_dict(st)
+    # reference init: zero biases, small heads (connect6/model.py:83-94)
+    fresh = c6.PolicyValueNet()
+    assert all(torch.count_nonzero(c.bias) == 0 for c in fresh.convs)
+    assert torch.count_nonzero(fresh.policy_output.bias) == 0
+    assert fresh.policy_output.weight.std() < 0.02 and fresh.value_output.weight.std() < 0.02
+    assert abs(fresh.convs[7].weight.std().item() / (2.0 / 864) ** 0.5 - 1) < 0.05
+
+
+def test_constructor_validation():
+    for bad in (
+        dict(kernels=[3, 3], channels=[8]),
+        dict(kernels=[], channels=[]),
+        dict(kernels=[2], channels=[8]),
+        dict(kernels=[-1], channels=[8]),
+        dict(kernels=[3], channels=[0]),
+    ):
+        with pytest.raises(ValueError):
+            c6.PolicyValueNet(board_size=5, **bad)
+    small = c6.PolicyValueNet(board_size=5, kernels=[3, 3, 3], channels=[8, 8, 16])
+    assert small.receptive_field == 7 and not small.is_default_architecture
+
+
+def test_forward_errors():
+    model = c6.PolicyValueNet()
+    with pytest.raises(ValueError):          # shape errors first, as connect6/model.py:97-102
+        model(torch.zeros(2, 4, 19, 19))
+    with pytest.raises(ValueError):
+        model(torch.zeros(3, 19, 19))
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        with torch.no_grad():
+            model(torch.zeros(2, 3, 19, 19))
+    model.precision = "int4"
+    with pytest.raises(ValueError):
+        model.resolve_precision()
+
+
+def test_precision_resolution_follows_torch_rules():
+    model = c6.PolicyValueNet()
+    assert model.resolve_precision() == _lib.PREC_F32
+    model.precision = "bf16x2"
+    assert model.resolve_precision() == _lib.PREC_BF16X2
+    model.precision = None
+    assert model.to(torch.bfloat16).resolve_precision() == _lib.PREC_BF16
+
+
+def test_mask_logits_argument_checks():
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        c6.mask_logits(torch.zeros(2, 361), torch.ones(2, 361, dtype=torch.bool))
+
+
+def _checkpoints(n, **kw):
+    cfg = {"architecture_version": 4, "kernels": list(R.DEFAULT_KERNELS),
+           "channels": list(R.DEFAULT_CHANNELS), "compile": False, "compile_mode": "default"}
+    return [
+        c6.HistoricalCheckpoint(path=Path(f"model_update_{i + 1:08d}.pt"), update=i + 1,
+                                model_state=R.init_state(50 + i, "reference"),
+                                model_config=dict(cfg, **kw), game_config={"board_size": 19, "win_length": 6})
+        for i in range(n)
+    ]
+
+
+def test_history_ensemble_construction_and_validation():
+    with pytest.raises(ValueError):
+        c6.HistoricalPolicyEnsemble([], torch.device("cpu"))
+    cps = _checkpoints(2)
+    ens = c6.HistoricalPolicyEnsemble(cps, torch.device("cpu"))
+    assert ens.num_models == 2 and ens.updates == [1, 2] and ens.board_size == 19
+    assert ens.kernels == R.DEFAULT_KERNELS and ens.channels == R.DEFAULT_CHANNELS
+    assert ens.action_size == 361 and ens.input_channels == 3 and ens.dtype == torch.float32
+    assert ens.conv_weights[0].shape == (2, 32, 3, 23, 23)
+    assert ens.conv_biases[7].shape == (2, 96)
+    assert ens.policy_weight.shape == (2, 1, 96, 1, 1) and ens.policy_bias.shape == (2, 1)
+    # compile keys are ignored when comparing architectures (history.py:69-73)
+    cps[1].model_config["compile"] = True
+    c6.HistoricalPolicyEnsemble(cps, torch.device("cpu"))
+    bad = _checkpoints(2)
+    bad[1].game_config = {"board_size": 15}
+    with pytest.raises(ValueError):
+        c6.HistoricalPolicyEnsemble(bad, torch.device("cpu"))
+    bad = _checkpoints(2)
+    bad[1].model_config["channels"] = [32] * 8
+    with pytest.raises(ValueError):
+        c6.HistoricalPolicyEnsemble(bad, torch.device("cpu"))
+    bad = _checkpoints(2)
+    del bad[1].model_state["convs.3.weight"]
+    with pytest.raises(KeyError):
+        c6.HistoricalPolicyEnsemble(bad, torch.device("cpu"))
+    with pytest.raises(ValueError):   # shape errors as history.py:277-286
+        ens.forward_grouped(torch.zeros(2, 3, 19, 19))
+    with pytest.raises(ValueError):
+        ens.forward_grouped(torch.zeros(3, 4, 3, 19, 19))
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        ens.forward_grouped(torch.zeros(2, 4, 3, 19, 19))
+
+
+def test_symmetry_helpers_on_host():
+    # tests/test_training_features.py:154-187 and tests/test_model.py:40-53 of the reference
+    want = [(0, False), (1, False), (2, False), (3, False), (0, True), (1, True), (2, True), (3, True)]
+    assert [c6.symmetry_for_phase(i) for i in range(8)] == want
+    assert c6.symmetry_for_phase(8) == want[0]
+    board = torch.arange(9, dtype=torch.int8).reshape(1, 3, 3)
+    actions = torch.arange(9, dtype=torch.long)
+    for phase in range(8):
+        k, flip = c6.symmetry_for_phase(phase)
+        tb = c6.transform_boards(board, k, flip)
+        ta = c6.transform_actions(actions, 3, k, flip)
+        assert torch.equal(tb.reshape(-1)[ta], board.reshape(-1)[actions])
+        assert torch.equal(c6.inverse_transform_actions(ta, board_size=3, k=k, flip=flip), actions)
+        assert torch.equal(tb, R.transform_boards(board, k, flip))
+    n = 7
+    b = torch.zeros(1, n, n, dtype=torch.int8)
+    b[0, 1, 2] = 1
+    a = torch.tensor([1 * n + 2])
+    for k in range(4):
+        for flip in (False, True):
+            ob, oa = c6.transform_boards(b, k, flip), int(c6.transform_actions(a, n, k, flip))
+            assert int(ob[0, oa // n, oa % n]) == 1
+            assert torch.equal(c6.inverse_transform_actions(torch.tensor([oa]), n, k, flip), a)

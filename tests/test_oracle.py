@@ -1,0 +1,244 @@
+"""Pins the CPU oracle (oracle/) without any GPU: brute force, closed forms,
+known answers and the reference's own invariants."""
+import math
+
+import pytest
+import torch
+
+from connect6_amd.synthetic import gen_boards, gen_uniform
+from oracle import cref
+from oracle import torch_ref as R
+
+TINY = dict(kernels=(3, 3, 3), channels=(8, 8, 16))  # tests/test_training_features.py:122-129
+
+
+def test_init_state_keys_shapes_and_scale():
+    st = R.init_state(0, "reference")
+    assert len(st) == 20
+    cin = 3
+    for i, (k, c) in enumerate(zip(R.DEFAULT_KERNELS, R.DEFAULT_CHANNELS)):
+        assert st[f"convs.{i}.weight"].shape == (c, cin, k, k)
+        assert st[f"convs.{i}.bias"].shape == (c,)
+        assert torch.count_nonzero(st[f"convs.{i}.bias"]) == 0
+        want = math.sqrt(2.0 / (cin * k * k))
+        assert abs(st[f"convs.{i}.weight"].std().item() / want - 1) < 0.05
+        cin = c
+    assert st["policy_output.weight"].shape == (1, 96, 1, 1)
+    assert st["value_output.weight"].shape == (1, 96, 1, 1)
+    assert abs(st["policy_output.weight"].std().item() / 0.01 - 1) < 0.3
+    n_params = sum(v.numel() for v in st.values())
+    assert n_params == 374082
+    td = R.init_state(0, "torch_default")
+    assert td["convs.3.bias"].abs().max() <= 1 / math.sqrt(64 * 9)
+
+
+def test_forward_matches_bruteforce_c_tiny():
+    st = R.init_state(5, "torch_default", **TINY)
+    x = torch.randn(3, 3, 5, 5, generator=torch.Generator().manual_seed(1))
+    lt, vt = R.forward(st, x)
+    lc, vc = cref.forward(st, x)
+    assert lt.shape == (3, 25) and vt.shape == (3,)
+    assert torch.allclose(lt, lc, atol=1e-6, rtol=1e-5)
+    assert torch.allclose(vt, vc, atol=1e-6, rtol=1e-5)
+
+
+def test_forward_matches_bruteforce_c_default_architecture():
+    st = R.init_state(1234, "torch_default")
+    x, _ = gen_boards(2, 200, 11)
+    lt, vt = R.forward(st, x)
+    lc, vc = cref.forward(st, x)
+    assert float((lt - lc).norm() / lc.norm()) < 1e-5
+    assert torch.allclose(vt, vc, atol=1e-6)
+
+
+def test_forward_one_layer_hand_computed():
+    # 1x1 conv with weight 2 and bias 1 on a single plane, heads = identity / 0.5
+    st = {
+        "convs.0.weight": torch.tensor([[[[2.0]], [[0.0]], [[0.0]]]]),
+        "convs.0.bias": torch.tensor([1.0]),
+        "policy_output.weight": torch.tensor([[[[1.0]]]]),
+        "policy_output.bias": torch.tensor([0.25]),
+        "value_output.weight": torch.tensor([[[[0.5]]]]),
+        "value_output.bias": torch.tensor([0.0]),
+    }
+    x = torch.zeros(1, 3, 2, 2)
+    x[0, 0] = torch.tensor([[0.0, 1.0], [2.0, -1.0]])
+    z = 2 * x[0, 0] + 1
+    a = z / (1 + torch.exp(-z))
+    logits, value = R.forward(st, x)
+    assert torch.allclose(logits, (a + 0.25).reshape(1, 4))       # row-major flatten
+    assert torch.allclose(value, torch.tanh((0.5 * a).mean()).reshape(1))
+
+
+def test_zero_input_known_answer_and_value_range():
+    st = R.init_state(3, "reference")
+    logits, value = R.forward(st, torch.zeros(3, 3, 19, 19))      # tests/test_model.py:13-17
+    assert logits.shape == (3, 361) and value.shape == (3,)
+    assert torch.count_nonzero(logits) == 0 and torch.count_nonzero(value) == 0
+    x, _ = gen_boards(16, 200, 2)
+    _, v = R.forward(R.init_state(3, "torch_default"), x)
+    assert torch.all(v <= 1) and torch.all(v >= -1)
+
+
+def test_forward_rejects_bad_shape():
+    st = R.init_state(3, "reference")
+    with pytest.raises(ValueError):
+        R.forward(st, torch.zeros(3, 2, 19, 19))
+    with pytest.raises(ValueError):
+        R.forward(st, torch.zeros(3, 19, 19))
+
+
+def test_grouped_equals_individual_models():
+    # the reference's invariant, tests/test_training_features.py:120-151
+    states = [R.init_state(100 + i, "reference", **TINY) for i in range(2)]
+    x = torch.randn(2, 5, 3, 5, 5, generator=torch.Generator().manual_seed(123))
+    grouped = R.forward_grouped(states, x)
+    assert grouped.shape == (2, 5, 25)
+    for i, s in enumerate(states):
+        assert torch.allclose(grouped[i], R.forward(s, x[i])[0], atol=1e-5, rtol=1e-5)
+    states = [R.init_state(7 + i, "torch_default") for i in range(2)]
+    xb, _ = gen_boards(4, 200, 5)
+    xg = xb.view(2, 2, 3, 19, 19)
+    assert torch.allclose(R.forward_grouped(states, xg), R.forward_grouped_loop(states, xg), atol=1e-5)
+    with pytest.raises(ValueError):
+        R.forward_grouped([], xg)
+
+
+def test_mask_logits_bit_patterns():
+    logits = torch.randn(4, 361)
+    _, legal = gen_boards(4, 200, 9)
+    out = R.mask_logits(logits, legal)
+    lowest = torch.tensor(torch.finfo(torch.float32).min)
+    assert torch.equal(out[~legal].view(torch.int32), lowest.view(torch.int32).expand(int((~legal).sum())))
+    assert torch.equal(out[legal].view(torch.int32), logits[legal].view(torch.int32))
+    assert torch.all(torch.isneginf(R.mask_logits(logits, legal, float("-inf"))[~legal]))
+    x, lg = gen_boards(4, 200, 9)
+    assert torch.equal(R.legal_from_input(x), lg)
+
+
+def _sample_loop(logits, legal, u, temperature):
+    out = []
+    for b in range(logits.shape[0]):
+        z = [(logits[b, i].item() / max(temperature, 1e-4)) if legal[b, i] else -math.inf for i in range(logits.shape[1])]
+        m = max(z)
+        e = [math.exp(v - m) for v in z]
+        total = sum(e)
+        run, pick = 0.0, None
+        for i, v in enumerate(e):
+            run += v
+            if legal[b, i] and run > u[b].item() * total:
+                pick = i
+                break
+        if pick is None:
+            pick = max(i for i in range(len(z)) if legal[b, i])
+        out.append((pick, z[pick] - m - math.log(total)))
+    return out
+
+
+def test_sample_inverse_cdf_matches_python_loop_and_respects_mask():
+    g = torch.Generator().manual_seed(4)
+    logits = torch.randn(64, 361, generator=g) * 2
+    _, legal = gen_boards(64, 300, 17)
+    u = gen_uniform(64, 3)
+    a, lp = R.sample_inverse_cdf(logits, legal, u, 0.7)
+    want = _sample_loop(logits, legal, u, 0.7)
+    assert [int(v) for v in a] == [w[0] for w in want]
+    assert torch.allclose(lp, torch.tensor([w[1] for w in want], dtype=torch.float32), atol=1e-4)
+    assert bool(legal.gather(1, a.view(-1, 1)).all())
+    # u -> 1 picks the last legal square, u = 0 the first with non-zero mass
+    a1, _ = R.sample_inverse_cdf(logits, legal, torch.full((64,), 0.99999994), 1.0)
+    assert bool(legal.gather(1, a1.view(-1, 1)).all())
+    a0, _ = R.sample_inverse_cdf(logits, legal, torch.zeros(64), 1.0)
+    assert torch.equal(a0, legal.float().argmax(1))
+
+
+def test_sample_inverse_cdf_distribution():
+    logits = torch.tensor([[0.0, 1.0, 2.0, -1.0] + [0.0] * 357])
+    legal = torch.zeros(1, 361, dtype=torch.bool)
+    legal[0, :4] = True
+    legal[0, 2] = False
+    n = 20000
+    u = torch.rand(n, generator=torch.Generator().manual_seed(0))
+    a, _ = R.sample_inverse_cdf(logits.expand(n, -1), legal.expand(n, -1), u, 1.0)
+    p = torch.softmax(torch.tensor([0.0, 1.0, -1.0]), 0)
+    freq = torch.tensor([(a == 0).float().mean(), (a == 1).float().mean(), (a == 3).float().mean()])
+    assert int((a == 2).sum()) == 0 and int((a > 3).sum()) == 0
+    assert torch.allclose(freq, p, atol=0.015)
+
+
+def test_symmetry_cycle_order():
+    # tests/test_training_features.py:154-166
+    want = [(0, False), (1, False), (2, False), (3, False), (0, True), (1, True), (2, True), (3, True)]
+    assert [R.symmetry_for_phase(i) for i in range(8)] == want
+    assert R.symmetry_for_phase(8) == want[0]
+
+
+@pytest.mark.parametrize("n", [3, 7, 19])
+def test_d4_maps_match_rot90_flip_and_invert(n):
+    board = torch.arange(n * n, dtype=torch.int64).reshape(1, n, n)
+    actions = torch.arange(n * n)
+    for phase in range(8):
+        k, flip = R.symmetry_for_phase(phase)
+        lib = torch.rot90(board, k=k, dims=(-2, -1)) if k else board      # train.py:228-230
+        lib = torch.flip(lib, dims=(-1,)) if flip else lib
+        view = R.transform_boards(board, k, flip)
+        assert torch.equal(view, lib)
+        ta = R.transform_actions(actions, n, k, flip)
+        # tests/test_training_features.py:169-187: a stone stays under its transformed action
+        assert torch.equal(view.reshape(-1)[ta], board.reshape(-1)[actions])
+        assert torch.equal(R.inverse_transform_actions(ta, n, k, flip), actions)
+        assert sorted(ta.tolist()) == list(range(n * n))
+
+
+def test_d4_single_stone_follows_action():
+    # tests/test_model.py:40-53
+    n = 7
+    board = torch.zeros(1, n, n, dtype=torch.int8)
+    board[0, 1, 2] = 1
+    action = torch.tensor([1 * n + 2])
+    for k in range(4):
+        for flip in (False, True):
+            ob = R.transform_boards(board, k, flip)
+            oa = int(R.transform_actions(action, n, k, flip))
+            assert int(ob[0, oa // n, oa % n]) == 1
+            assert torch.equal(R.inverse_transform_actions(torch.tensor([oa]), n, k, flip), action)
+
+
+def test_d4_average_recovers_equivariant_map():
+    base = torch.randn(5, 361)
+    vals = torch.randn(8, 5)
+    views = R.d4_expand(base.view(5, 1, 19, 19)).view(8, 5, 361)   # view p shows base through D4 map p
+    logits, values = R.d4_average(views, vals)
+    assert torch.allclose(logits, base, atol=1e-6)
+    assert torch.allclose(values, vals.mean(0))
+    # brute force for one entry
+    b, a = 2, 123
+    s = sum(views[p, b, int(R.transform_actions(torch.tensor([a]), 19, *R.symmetry_for_phase(p)))] for p in range(8))
+    assert abs(float(s) / 8 - float(logits[b, a])) < 1e-6
+
+
+def test_bf16_emulation_is_close_to_fp32():
+    st = R.init_state(1234, "reference")
+    x, legal = gen_boards(64, 200, 2025)
+    l32, v32 = R.forward(st, x)
+    l16, v16 = R.forward_bf16_emulated(st, x)
+    assert float((l16 - l32).norm() / l32.norm()) < 2e-2
+    assert float((v16 - v32).norm() / v32.norm()) < 2e-2
+
+
+def test_generator_properties():
+    x, legal = gen_boards(512, 200, 2025)
+    assert x.shape == (512, 3, 19, 19) and x.dtype == torch.float32
+    assert set(torch.unique(x).tolist()) <= {0.0, 1.0}
+    own, opp = x[:, 0].flatten(1).sum(1), x[:, 1].flatten(1).sum(1)
+    assert float((x[:, 0] * x[:, 1]).sum()) == 0            # no overlaps
+    assert torch.all((opp - own == 0) | (opp - own == 1))    # split as evenly as possible
+    assert int((own + opp).max()) <= 200 and int((own + opp).min()) >= 0
+    plane = x[:, 2].flatten(1)
+    assert torch.all((plane.min(1).values == plane.max(1).values))
+    assert 0.35 < float(plane[:, 0].mean()) < 0.65
+    assert torch.equal(legal, (x[:, 0] + x[:, 1] == 0).flatten(1))
+    x2, _ = gen_boards(512, 200, 2025)
+    assert torch.equal(x, x2)
+    x3, _ = gen_boards(64, 300, 1)
+    assert int((x3[:, 0] + x3[:, 1]).flatten(1).sum(1).max()) > 200
