@@ -1,0 +1,225 @@
+#!/usr/bin/env python3
+"""Headline benchmark: boards/s of the B=4096 16-bit forward on one MI355X.
+
+One "step" is one batched forward of 4096 synthetic positions through the
+default-architecture policy/value CNN (inputs and packed weights already in
+HBM).  Prints ONE JSON line.  Alongside the headline it reports the fused
+kernel's MFMA roofline fraction (HIP-event timing of the kernel launches), the
+G=8 grouped-history rate, the other arithmetic modes with their agreement with
+the fp32 kernel, the HBM-bound tail kernels, and a CPU baseline (the PyTorch
+oracle on the host cores, bounded sample).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+CONV_FLOP_PER_BOARD = 269_554_368        # dense conv count, 2 * 134,777,184 MAC
+MFMA_PEAK_TFLOPS = 2500.0                # MI355X dense bf16 / fp16
+HBM_PEAK_GBS = 8000.0
+HEADLINE = "bf16x2"                      # bf16 MFMA mode that meets the >= 99 % argmax gate
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--batch", type=int, default=4096)
+    ap.add_argument("--precision", default=HEADLINE, choices=["bf16x2", "bf16", "fp16", "fp32"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true", help="headline + roofline only")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: the forward shards by board with no exchange step, "
+              "and this build runs and reports a single MI355X only (use --gpus 1).", file=sys.stderr)
+        return 2
+
+    import torch
+
+    import connect6_amd as c6
+    from connect6_amd.synthetic import gen_boards, gen_uniform
+
+    dev = torch.device("cuda:0")
+    c6.load()
+    B, K, W = args.batch, args.steps, args.warmup
+    torch.manual_seed(1234)
+    model = c6.PolicyValueNet().to(dev).eval()       # reference init (connect6/model.py:83-94)
+    x_host, legal_host = gen_boards(B, 200, 2025)
+    x = x_host.to(dev)
+    legal = legal_host.to(dev)
+
+    def run_mode(prec: str, steps: int, warmup: int):
+        """(seconds per step by wall clock, seconds per launch by HIP events)"""
+        model.precision = prec
+        with torch.inference_mode():
+            for _ in range(warmup):
+                model.forward_masked(x, fill=float("-inf"))
+            torch.cuda.synchronize()
+            evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+                   for _ in range(steps)]
+            t0 = time.perf_counter()
+            for a, b in evs:
+                a.record()                         # same stream the kernel is launched on
+                model.forward_masked(x, fill=float("-inf"))
+                b.record()
+            torch.cuda.synchronize()
+            wall = (time.perf_counter() - t0) / steps
+        kernel = sum(a.elapsed_time(b) for a, b in evs) / steps * 1e-3
+        return wall, kernel
+
+    wall, kern = run_mode(args.precision, K, W)
+    value = B / wall
+    achieved = B * CONV_FLOP_PER_BOARD / kern / 1e12
+    out = {
+        "metric": "boards/sec B=4096 16-bit forward (masked logits + value), 1x MI355X",
+        "value": value,
+        "unit": "boards/s",
+        "n_gpus": 1,
+        "steps": K,
+        "warmup": W,
+        "ms_per_step": wall * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"configs[1]: default CNN, B={B}, stones 0..200, masked logits + value, "
+                        f"reference init, seed 1234/2025",
+            "precision_mode": args.precision,
+            "batch": B,
+        },
+        "roofline": {
+            "bound": "mfma",
+            "achieved": achieved,
+            "peak": MFMA_PEAK_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": achieved / MFMA_PEAK_TFLOPS,
+            "traffic": None,
+            "kernel": "fused_forward_kernel",
+            "kernel_ms": kern * 1e3,
+            "flop_per_board": CONV_FLOP_PER_BOARD,
+        },
+    }
+
+    if not args.no_extras:
+        # ---- every arithmetic mode, with its agreement with the fp32 kernel ----
+        model.precision = "fp32"
+        with torch.inference_mode():
+            l32, v32 = model.forward_masked(x, fill=float("-inf"))
+        modes = {}
+        for prec in ("bf16x2", "bf16", "fp16", "fp32"):
+            w_, k_ = run_mode(prec, max(5, K // 2), 3)
+            with torch.inference_mode():
+                lg, vg = model.forward_masked(x, fill=float("-inf"))
+            fin = torch.isfinite(l32)
+            modes[prec] = {
+                "boards_per_s": B / w_,
+                "kernel_ms": k_ * 1e3,
+                "mfma_frac_dense": B * CONV_FLOP_PER_BOARD / k_ / 1e12 / (157.3 if prec == "fp32" else MFMA_PEAK_TFLOPS),
+                "rel_l2_logits_vs_fp32_kernel": float((lg[fin] - l32[fin]).norm() / l32[fin].norm()),
+                "argmax_agreement_vs_fp32_kernel": float((lg.argmax(1) == l32.argmax(1)).float().mean()),
+            }
+        out["modes"] = modes
+
+        # ---- grouped history: G=8 weight sets x 512 boards in one launch (configs[2]) ----
+        cfg = {"architecture_version": 4, "kernels": list(model.kernels), "channels": list(model.channels)}
+        cps = []
+        for i in range(8):
+            torch.manual_seed(1234 + i)
+            cps.append(c6.HistoricalCheckpoint(
+                path=Path(f"model_update_{i + 1:08d}.pt"), update=i + 1,
+                model_state=c6.PolicyValueNet().state_dict(), model_config=cfg,
+                game_config={"board_size": 19, "win_length": 6}))
+        ens = c6.HistoricalPolicyEnsemble(cps, dev, dtype=torch.bfloat16,
+                                          precision=None if args.precision == "fp32" else args.precision)
+        xg = x.view(8, B // 8, 3, 19, 19).to(torch.bfloat16)
+
+        def timed(fn, steps=max(5, K // 2), warmup=3):
+            with torch.inference_mode():
+                for _ in range(warmup):
+                    fn()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(steps):
+                    fn()
+                torch.cuda.synchronize()
+            return (time.perf_counter() - t0) / steps
+
+        tg = timed(lambda: ens.forward_grouped(xg))
+        out["grouped_g8"] = {
+            "boards_per_s": B / tg, "ms": tg * 1e3, "ratio_to_single": (B / tg) / value,
+            "workload": f"configs[2]: 8 weight sets x {B // 8} boards, one launch, bf16 in/out",
+        }
+
+        # ---- fused self-play step, configs[3]: B=16384, stones 0..300 ----
+        model.precision = args.precision
+        xs = gen_boards(16384, 300, 2025)[0].to(dev)
+        us = gen_uniform(16384, 7).to(dev)
+        ts = timed(lambda: model.selfplay_step(xs, us, 1.0), steps=10)
+        out["selfplay_step_b16384"] = {"boards_per_s": 16384 / ts, "ms": ts * 1e3}
+
+        # ---- D4-averaged evaluation, configs[4]: 8192 base boards -> 65536 views ----
+        xd = gen_boards(8192, 200, 2025)[0].to(dev)
+        td = timed(lambda: c6.evaluate_d4(model, xd), steps=5, warmup=2)
+        out["d4_eval_8192x8"] = {"base_boards_per_s": 8192 / td, "ms": td * 1e3}
+
+        # ---- HBM-bound tail kernels: algorithmic bytes / time ----
+        nb = 65536
+        lg = torch.randn(nb, 361, device=dev)
+        lgl = gen_boards(nb, 300, 5)[1].to(dev)
+        un = gen_uniform(nb, 3).to(dev)
+        views = torch.randn(8, 8192, 361, device=dev)
+        vals = torch.randn(8, 8192, device=dev)
+        hbm = {}
+        t = timed(lambda: c6.mask_logits(lg, lgl), steps=20)
+        hbm["mask_logits_f32"] = {"GBps": nb * 361 * (4 + 1 + 4) / t / 1e9}
+        t = timed(lambda: c6.sample_actions(lg, lgl, 1.0, un), steps=20)
+        hbm["softmax_sample"] = {"GBps": nb * (361 * 5 + 4 + 12) / t / 1e9}
+        t = timed(lambda: c6.d4_expand(xd), steps=20)
+        hbm["d4_expand_f32"] = {"GBps": 8192 * 3 * 361 * 4 * 9 / t / 1e9}
+        t = timed(lambda: c6.d4_reduce(views, vals), steps=20)
+        hbm["d4_reduce"] = {"GBps": 8192 * (361 * 4 * 9 + 4 * 9) / t / 1e9}
+        for v in hbm.values():
+            v["frac_of_hbm_peak"] = v["GBps"] / HBM_PEAK_GBS
+        out["hbm_kernels"] = hbm
+
+    if not args.no_cpu_baseline:
+        # The PyTorch fp32 oracle (the checker) on this box's host cores, configs[0] shape.
+        from oracle import torch_ref as R
+
+        threads = min(os.cpu_count() or 1, 16)
+        torch.set_num_threads(threads)
+        st = {k: v.detach().cpu().float() for k, v in model.state_dict().items()}
+        xb = x_host[:256]
+        with torch.inference_mode():
+            for _ in range(2):
+                R.forward(st, xb)
+            times = []
+            t_end = time.perf_counter() + 12.0
+            while len(times) < 5 or (time.perf_counter() < t_end and len(times) < 40):
+                t0 = time.perf_counter()
+                R.forward(st, xb)
+                times.append(time.perf_counter() - t0)
+        times.sort()
+        med = times[len(times) // 2]
+        out["cpu_baseline"] = {
+            "value": 256 / med, "unit": "boards/s", "cores": threads, "kind": "port",
+            "sample": f"configs[0]: {len(times)} fp32 forwards of B=256 (same generator, same weights) "
+                      f"with the PyTorch oracle, median",
+        }
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

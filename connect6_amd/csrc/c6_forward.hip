@@ -113,19 +113,30 @@ __device__ __forceinline__ void conv1_accumulate(const unsigned char *smem,
   v4i ring[D];
 #pragma unroll
   for (int d = 0; d < D; ++d) ring[d] = wl[d * 64];
+  v4i bcur[3];
+#pragma unroll
+  for (int j = 0; j < 3; ++j) bcur[j] = *reinterpret_cast<const v4i *>(smem + l1base[j]);
 #pragma unroll 1
   for (int it = 0; it < ITERS; ++it) {
     const int adv = it * ROWS_BODY * ROWB;
     const v4i *wn = wl + (size_t)(it * U + D) * 64;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int off = (u / CPR) * ROWB + (u % CPR) * 16;
-      v4i b[3];
+      // operand fragments of the NEXT k-step are fetched while this step's MFMAs run; after
+      // the last step this reads the zero row / next copy, which is harmless
+      const int un = u + 1;
+      const int offn = (un / CPR) * ROWB + (un % CPR) * 16;
+      v4i bnext[3];
 #pragma unroll
-      for (int j = 0; j < 3; ++j) b[j] = *reinterpret_cast<const v4i *>(smem + l1base[j] + adv + off);
+      for (int j = 0; j < 3; ++j)
+        bnext[j] = *reinterpret_cast<const v4i *>(smem + l1base[j] + adv + offn);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int j = 0; j < 3; ++j) mma<P>(ring[u % D], b[j], acc[0][j]);
-      ring[u % D] = wn[u * 64];  // prefetch k-step (it*U + u + D); the tail over-reads zero frags
+      for (int j = 0; j < 3; ++j) mma<P>(ring[u % D], bcur[j], acc[0][j]);
+      ring[u % D] = wn[u * 64];  // prefetch k-step (it*U + u + D); the tail over-reads the next layer
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int j = 0; j < 3; ++j) bcur[j] = bnext[j];
     }
   }
 }
@@ -150,77 +161,107 @@ __device__ __forceinline__ void conv3_accumulate(const unsigned char *smem,
 #pragma unroll
     for (int t = 0; t < NT; ++t) ring[d][t] = wl[(d * NT + t) * 64];
 
+  auto tap_base = [&](int j, int ky, int kx) {
+    const int pp = ci[j] + (ky - 1) * kPitch + (kx - 1);
+    return pp * G::PIXB + (((h ^ (pp >> 2)) & 1) << 4);
+  };
+  int base[3][3];
+#pragma unroll
+  for (int j = 0; j < 3; ++j)
+#pragma unroll
+    for (int kx = 0; kx < 3; ++kx) base[j][kx] = tap_base(j, 0, kx);
+  v4i bcur[3], lcur[3];
+#pragma unroll
+  for (int j = 0; j < 3; ++j) {
+    bcur[j] = *reinterpret_cast<const v4i *>(smem + base[j][0]);
+    if constexpr (P::SPLIT) lcur[j] = *reinterpret_cast<const v4i *>(smem + base[j][0] + G::PLANE);
+  }
+
 #pragma unroll 1
   for (int ky = 0; ky < 3; ++ky) {
-    int base[3][3];
+    int nbase[3][3];  // next kernel row (wraps to row 0 after the last: one harmless extra fetch)
+    const int kyn = ky == 2 ? 0 : ky + 1;
 #pragma unroll
     for (int j = 0; j < 3; ++j)
 #pragma unroll
-      for (int kx = 0; kx < 3; ++kx) {
-        const int pp = ci[j] + (ky - 1) * kPitch + (kx - 1);
-        base[j][kx] = pp * G::PIXB + (((h ^ (pp >> 2)) & 1) << 4);
-      }
+      for (int kx = 0; kx < 3; ++kx) nbase[j][kx] = tap_base(j, kyn, kx);
     const v4i *wn = wl + (size_t)(ky * U + D) * NT * 64;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int kx = u / KC, kc = u % KC;
-      v4i b[3];
+      // fetch the activation fragments of the next k-step while this step's MFMAs run
+      v4i bnext[3], lnext[3];
 #pragma unroll
-      for (int j = 0; j < 3; ++j) b[j] = *reinterpret_cast<const v4i *>(smem + base[j][kx] + kc * 32);
+      for (int j = 0; j < 3; ++j) {
+        const int a = (u + 1 < U) ? base[j][(u + 1) / KC] + ((u + 1) % KC) * 32 : nbase[j][0];
+        bnext[j] = *reinterpret_cast<const v4i *>(smem + a);
+        if constexpr (P::SPLIT) lnext[j] = *reinterpret_cast<const v4i *>(smem + a + G::PLANE);
+      }
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int t = 0; t < NT; ++t)
 #pragma unroll
-        for (int j = 0; j < 3; ++j) mma<P>(ring[u % D][t], b[j], acc[t][j]);
+        for (int j = 0; j < 3; ++j) mma<P>(ring[u % D][t], bcur[j], acc[t][j]);
       if constexpr (P::SPLIT) {
-        v4i bl[3];
-#pragma unroll
-        for (int j = 0; j < 3; ++j)
-          bl[j] = *reinterpret_cast<const v4i *>(smem + base[j][kx] + kc * 32 + G::PLANE);
 #pragma unroll
         for (int t = 0; t < NT; ++t)
 #pragma unroll
-          for (int j = 0; j < 3; ++j) mma<P>(ring[u % D][t], bl[j], acc[t][j]);
+          for (int j = 0; j < 3; ++j) mma<P>(ring[u % D][t], lcur[j], acc[t][j]);
       }
+      // weights of k-step u+D replace the ones just consumed (the tail over-reads the next layer)
 #pragma unroll
       for (int t = 0; t < NT; ++t) ring[u % D][t] = wn[(u * NT + t) * 64];
-    }
-  }
-}
-
-// bias + SiLU + store of one layer's accumulators into the activation tile
-template <class P, int COUT>
-__device__ __forceinline__ void store_activations(unsigned char *smem,
-                                                  const float *__restrict__ bias,
-                                                  const int (&ci)[3], const bool (&valid)[3],
-                                                  int h, const f32x16 (&acc)[COUT / 32][3]) {
-  using G = Geo<P>;
-  constexpr int NT = COUT / 32;
-#pragma unroll
-  for (int t = 0; t < NT; ++t)
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int ch0 = 32 * t + 8 * q + 4 * h;
-      const f32x4 b4 = *reinterpret_cast<const f32x4 *>(bias + ch0);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int j = 0; j < 3; ++j) {
-        if (valid[j]) {
-          float v[4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) v[e] = silu<P>(acc[t][j][4 * q + e] + b4[e]);
-          const int off = ci[j] * G::PIXB + ((ch0 * G::EB) ^ (((ci[j] >> 2) & 1) << 4));
-          store4<P>(smem + off, v);
-        }
+        bcur[j] = bnext[j];
+        if constexpr (P::SPLIT) lcur[j] = lnext[j];
       }
     }
-}
-
-template <int N> __device__ __forceinline__ void zero_acc(f32x16 (&acc)[N][3]) {
-#pragma unroll
-  for (int t = 0; t < N; ++t)
 #pragma unroll
     for (int j = 0; j < 3; ++j)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) acc[t][j][i] = 0.0f;
+      for (int kx = 0; kx < 3; ++kx) base[j][kx] = nbase[j][kx];
+  }
+}
+
+// SiLU + store of one layer's accumulators (bias already added at init) into the
+// activation tile.  Lanes beyond pixel 360 shadow pixel 360 (same inputs, same
+// results, same address), so every lane stores unconditionally.
+template <class P, int COUT>
+__device__ __forceinline__ void store_activations(unsigned char *smem, const int (&ci)[3], int h,
+                                                  const f32x16 (&acc)[COUT / 32][3]) {
+  using G = Geo<P>;
+  constexpr int NT = COUT / 32;
+#pragma unroll
+  for (int j = 0; j < 3; ++j) {
+    const int pbase = ci[j] * G::PIXB;
+    const int swz = ((ci[j] >> 2) & 1) << 4;
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int ch0 = 32 * t + 8 * q + 4 * h;
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = silu<P>(acc[t][j][4 * q + e]);
+        store4<P>(smem + pbase + ((ch0 * G::EB) ^ swz), v);
+      }
+  }
+}
+
+// accumulators start at the layer's bias: lane (h) register i holds channel 32t + 8(i/4) + 4h + i%4
+template <int N>
+__device__ __forceinline__ void init_acc(f32x16 (&acc)[N][3], const float *__restrict__ bias, int h) {
+#pragma unroll
+  for (int t = 0; t < N; ++t)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const f32x4 b4 = *reinterpret_cast<const f32x4 *>(bias + 32 * t + 8 * q + 4 * h);
+#pragma unroll
+      for (int j = 0; j < 3; ++j)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[t][j][4 * q + e] = b4[e];
+    }
 }
 
 template <class P, int L, int CIN, int COUT>
@@ -229,11 +270,11 @@ __device__ __forceinline__ void mid_layer(unsigned char *smem, const unsigned ch
                                           const bool (&valid)[3], int h, int lane) {
   using G = Geo<P>;
   f32x16 acc[COUT / 32][3];
-  zero_acc(acc);
+  init_acc(acc, tail + bias_offset(L), h);
   const v4i *wl = reinterpret_cast<const v4i *>(packed + (size_t)G::frag_offset(L) * 1024) + lane;
   conv3_accumulate<P, CIN, COUT>(smem, wl, ci, h, acc);
   __syncthreads();  // every wave has finished reading the previous layer
-  store_activations<P, COUT>(smem, tail + bias_offset(L), ci, valid, h, acc);
+  store_activations<P, COUT>(smem, ci, h, acc);
   __syncthreads();
 }
 
@@ -311,7 +352,7 @@ __global__ __launch_bounds__(kThreads) void fused_forward_kernel(const FwdParams
     // ---- layer 1 ----
     {
       f32x16 acc[1][3];
-      zero_acc(acc);
+      init_acc(acc, tail + bias_offset(0), h);
       const v4i *wl = reinterpret_cast<const v4i *>(packed) + lane;
       conv1_accumulate<P>(smem, wl, l1base, acc);
       __syncthreads();
@@ -323,7 +364,7 @@ __global__ __launch_bounds__(kThreads) void fused_forward_kernel(const FwdParams
         const v4i z = {0, 0, 0, 0};
         *reinterpret_cast<v4i *>(smem + pos * G::PIXB + w16 * 16) = z;
       }
-      store_activations<P, 32>(smem, tail + bias_offset(0), ci, valid, h, acc);
+      store_activations<P, 32>(smem, ci, h, acc);
       __syncthreads();
     }
     mid_layer<P, 1, 32, 32>(smem, packed, tail, ci, valid, h, lane);
@@ -336,10 +377,9 @@ __global__ __launch_bounds__(kThreads) void fused_forward_kernel(const FwdParams
     // ---- layer 8 + both 1x1 heads straight from the fp32 accumulators ----
     {
       f32x16 acc[3][3];
-      zero_acc(acc);
+      init_acc(acc, tail + bias_offset(7), h);
       const v4i *wl = reinterpret_cast<const v4i *>(packed + (size_t)G::frag_offset(7) * 1024) + lane;
       conv3_accumulate<P, 96, 96>(smem, wl, ci, h, acc);
-      const float *bias = tail + bias_offset(7);
       const float *polw = tail + kBiasTotal;
       const float *valw = polw + kHeadC;
       float pol[3] = {0.0f, 0.0f, 0.0f};
@@ -349,14 +389,13 @@ __global__ __launch_bounds__(kThreads) void fused_forward_kernel(const FwdParams
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const int ch0 = 32 * t + 8 * q + 4 * h;
-          const f32x4 b4 = *reinterpret_cast<const f32x4 *>(bias + ch0);
           const f32x4 pw = *reinterpret_cast<const f32x4 *>(polw + ch0);
           const f32x4 vw = *reinterpret_cast<const f32x4 *>(valw + ch0);
 #pragma unroll
           for (int j = 0; j < 3; ++j)
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-              const float a = silu<P>(acc[t][j][4 * q + e] + b4[e]);
+              const float a = silu<P>(acc[t][j][4 * q + e]);
               pol[j] = fmaf(a, pw[e], pol[j]);
               const float va = a * vw[e];
               vsum += valid[j] ? va : 0.0f;
