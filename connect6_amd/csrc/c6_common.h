@@ -81,7 +81,13 @@ template <class P> struct Geo {
   static constexpr int E = 16 / EB;                 // elements per 16-byte fragment lane
   static constexpr int KSTEP = 2 * E;               // K elements contracted per fragment pair
   static constexpr int PLANE = kChSlots * EB;       // bytes of one precision plane of a position
-  static constexpr int PIXB = PLANE * (P::SPLIT ? 2 : 1);  // bytes per position
+  static constexpr int RECB = PLANE * (P::SPLIT ? 2 : 1);  // payload bytes per position
+  // LDS bank conflicts: a ds_read_b128 is served 16 lanes at a time, so 16 consecutive
+  // positions must land on 16 different 16-byte bank groups.  192-byte records get there
+  // with 16 bytes of padding (stride 208 = 13 x 16); 384-byte records (fp32, hi+lo) would
+  // not fit the LDS padded, so they XOR the 16-byte granule index with (position>>1)&7.
+  static constexpr bool PADDED = (EB == 2 && !P::SPLIT);
+  static constexpr int PIXB = PADDED ? RECB + 16 : RECB;  // bytes per position
   static constexpr int ACT_BYTES = kPos * PIXB;
   static constexpr int CPR = 24 / E;                // fragments per first-layer K row
   static constexpr int STEPS1 = kL1RowsHalf * CPR;  // first-layer k-steps

@@ -40,41 +40,56 @@ template <> __device__ __forceinline__ void mma<PrecF32>(const v4i &a, const v4i
   for (int e = 0; e < 4; ++e) c = __builtin_amdgcn_mfma_f32_32x32x2f32(af[e], bf[e], c, 0, 0, 0);
 }
 
-template <class P> __device__ __forceinline__ unsigned short bits16(float v);
-template <> __device__ __forceinline__ unsigned short bits16<PrecBF16>(float v) {
-  return __builtin_bit_cast(unsigned short, (__bf16)v);
-}
-template <> __device__ __forceinline__ unsigned short bits16<PrecBF16X2>(float v) {
-  return __builtin_bit_cast(unsigned short, (__bf16)v);
-}
-template <> __device__ __forceinline__ unsigned short bits16<PrecF16>(float v) {
-  return __builtin_bit_cast(unsigned short, (_Float16)v);
-}
-template <> __device__ __forceinline__ unsigned short bits16<PrecF32>(float) { return 0; }
-
-template <class P> __device__ __forceinline__ float from_bits16(unsigned short b);
-template <> __device__ __forceinline__ float from_bits16<PrecBF16X2>(unsigned short b) {
-  return __builtin_bit_cast(float, (unsigned)b << 16);
-}
-
-// store four consecutive channels of one position (dst already swizzled)
-template <class P> __device__ __forceinline__ void store4(unsigned char *dst, const float (&v)[4]) {
-  if constexpr (P::EB == 4) {
-    f32x4 o = {v[0], v[1], v[2], v[3]};
-    *reinterpret_cast<f32x4 *>(dst) = o;
+template <class P> __device__ __forceinline__ unsigned short bits16(float v) {
+  if constexpr (P::ID == C6_PREC_F16) {
+    return __builtin_bit_cast(unsigned short, (_Float16)v);
   } else {
-    v2i o;
-    o[0] = (int)((unsigned)bits16<P>(v[0]) | ((unsigned)bits16<P>(v[1]) << 16));
-    o[1] = (int)((unsigned)bits16<P>(v[2]) | ((unsigned)bits16<P>(v[3]) << 16));
-    *reinterpret_cast<v2i *>(dst) = o;
-    if constexpr (P::SPLIT) {
-      float r[4];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) r[e] = v[e] - from_bits16<P>(bits16<P>(v[e]));
+    return __builtin_bit_cast(unsigned short, (__bf16)v);  // RNE
+  }
+}
+
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+// two fp32 -> one dword of two 16-bit values (round to nearest even), low half first
+template <class P> __device__ __forceinline__ int pack2(float a, float b) {
+  const f32x2 v = {a, b};
+  if constexpr (P::ID == C6_PREC_F16) {
+    return __builtin_bit_cast(int, __builtin_convertvector(v, f16x2));
+  } else {
+    return __builtin_bit_cast(int, __builtin_convertvector(v, bf16x2));
+  }
+}
+__device__ __forceinline__ float bf16_lo(int w) { return __builtin_bit_cast(float, w << 16); }
+__device__ __forceinline__ float bf16_hi(int w) { return __builtin_bit_cast(float, w & (int)0xffff0000); }
+
+// XOR term of the granule swizzle for position `pos` (0 for the padded layout)
+template <class P> __device__ __forceinline__ int swz_of(int pos) {
+  if constexpr (Geo<P>::PADDED) {
+    return 0;
+  } else {
+    return ((pos >> 1) & 7) << 4;
+  }
+}
+
+// store four consecutive channels (logical byte offset `o` inside the record) of position `pos`
+template <class P>
+__device__ __forceinline__ void store4(unsigned char *smem, int pbase, int sw, int o,
+                                       const float (&v)[4]) {
+  if constexpr (P::EB == 4) {
+    const f32x4 w = {v[0], v[1], v[2], v[3]};
+    *reinterpret_cast<f32x4 *>(smem + pbase + (o ^ sw)) = w;
+  } else {
+    v2i w;
+    w[0] = pack2<P>(v[0], v[1]);
+    w[1] = pack2<P>(v[2], v[3]);
+    *reinterpret_cast<v2i *>(smem + pbase + (o ^ sw)) = w;
+    if constexpr (P::SPLIT) {  // low-order part: what the first rounding dropped
       v2i q;
-      q[0] = (int)((unsigned)bits16<P>(r[0]) | ((unsigned)bits16<P>(r[1]) << 16));
-      q[1] = (int)((unsigned)bits16<P>(r[2]) | ((unsigned)bits16<P>(r[3]) << 16));
-      *reinterpret_cast<v2i *>(dst + Geo<P>::PLANE) = q;
+      q[0] = pack2<P>(v[0] - bf16_lo(w[0]), v[1] - bf16_hi(w[0]));
+      q[1] = pack2<P>(v[2] - bf16_lo(w[1]), v[3] - bf16_hi(w[1]));
+      *reinterpret_cast<v2i *>(smem + pbase + ((o + Geo<P>::PLANE) ^ sw)) = q;
     }
   }
 }
@@ -83,7 +98,7 @@ template <class P> __device__ __forceinline__ float silu(float v) {
   if constexpr (P::EB == 4) {
     return v / (1.0f + expf(-v));
   } else {
-    return v * __builtin_amdgcn_rcpf(1.0f + __expf(-v));
+    return v * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(v * -1.4426950408889634f));
   }
 }
 
@@ -95,35 +110,56 @@ __device__ __forceinline__ float load_x(const void *x, int dt, size_t i) {
 }
 
 // ------------------------------------------------------------------------
+// weight-fragment prefetch rings.  A ring holds the fragments of the next
+// kRing k-steps; the ring of layer L+1 is loaded before the epilogue of layer
+// L so that no layer starts by waiting on L2.
+// ------------------------------------------------------------------------
+template <class P> struct L1Pipe {
+  static constexpr int CPR = Geo<P>::CPR;
+  static constexpr int ROWS_BODY = (CPR == 3) ? 7 : 1;
+  static constexpr int U = ROWS_BODY * CPR;
+  static constexpr int D = (CPR == 3) ? 7 : 6;
+  static constexpr int ITERS = kL1RowsHalf / ROWS_BODY;
+  static_assert(U % D == 0 && ITERS * ROWS_BODY == kL1RowsHalf, "first-layer pipeline shape");
+};
+
+template <int D, int NT>
+__device__ __forceinline__ void preload_ring(v4i (&ring)[D][NT], const v4i *__restrict__ wl) {
+#pragma unroll
+  for (int d = 0; d < D; ++d)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) ring[d][t] = wl[(d * NT + t) * 64];
+}
+
+template <class P, int L>
+__device__ __forceinline__ const v4i *layer_weights(const unsigned char *packed, int lane) {
+  return reinterpret_cast<const v4i *>(packed + (size_t)Geo<P>::frag_offset(L) * 1024) + lane;
+}
+
+// ------------------------------------------------------------------------
 // first layer: 23x23 on 3 planes, K = (ky, plane, kx24) split over lane halves
 // ------------------------------------------------------------------------
 template <class P>
 __device__ __forceinline__ void conv1_accumulate(const unsigned char *smem,
                                                  const v4i *__restrict__ wl,
+                                                 v4i (&ring)[L1Pipe<P>::D][1],
                                                  const int (&l1base)[3], f32x16 (&acc)[1][3]) {
   using G = Geo<P>;
-  constexpr int CPR = G::CPR;
+  using PP = L1Pipe<P>;
+  constexpr int CPR = PP::CPR, U = PP::U, D = PP::D;
   constexpr int ROWB = kL1RowPitch * G::EB;
-  constexpr int ROWS_BODY = (CPR == 3) ? 7 : 1;
-  constexpr int U = ROWS_BODY * CPR;
-  constexpr int D = (CPR == 3) ? 7 : 6;
-  constexpr int ITERS = kL1RowsHalf / ROWS_BODY;
-  static_assert(U % D == 0 && ITERS * ROWS_BODY == kL1RowsHalf, "first-layer pipeline shape");
 
-  v4i ring[D];
-#pragma unroll
-  for (int d = 0; d < D; ++d) ring[d] = wl[d * 64];
   v4i bcur[3];
 #pragma unroll
   for (int j = 0; j < 3; ++j) bcur[j] = *reinterpret_cast<const v4i *>(smem + l1base[j]);
 #pragma unroll 1
-  for (int it = 0; it < ITERS; ++it) {
-    const int adv = it * ROWS_BODY * ROWB;
+  for (int it = 0; it < PP::ITERS; ++it) {
+    const int adv = it * PP::ROWS_BODY * ROWB;
     const v4i *wn = wl + (size_t)(it * U + D) * 64;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       // operand fragments of the NEXT k-step are fetched while this step's MFMAs run; after
-      // the last step this reads the zero row / next copy, which is harmless
+      // the last step this reads the zero row / the next copy, which is harmless
       const int un = u + 1;
       const int offn = (un / CPR) * ROWB + (un % CPR) * 16;
       v4i bnext[3];
@@ -132,8 +168,8 @@ __device__ __forceinline__ void conv1_accumulate(const unsigned char *smem,
         bnext[j] = *reinterpret_cast<const v4i *>(smem + l1base[j] + adv + offn);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int j = 0; j < 3; ++j) mma<P>(ring[u % D], bcur[j], acc[0][j]);
-      ring[u % D] = wn[u * 64];  // prefetch k-step (it*U + u + D); the tail over-reads the next layer
+      for (int j = 0; j < 3; ++j) mma<P>(ring[u % D][0], bcur[j], acc[0][j]);
+      ring[u % D][0] = wn[u * 64];  // k-step (it*U + u + D); the tail over-reads the next layer
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int j = 0; j < 3; ++j) bcur[j] = bnext[j];
@@ -146,8 +182,10 @@ __device__ __forceinline__ void conv1_accumulate(const unsigned char *smem,
 // ------------------------------------------------------------------------
 template <class P, int CIN, int COUT>
 __device__ __forceinline__ void conv3_accumulate(const unsigned char *smem,
-                                                 const v4i *__restrict__ wl, const int (&ci)[3],
-                                                 int h, f32x16 (&acc)[COUT / 32][3]) {
+                                                 const v4i *__restrict__ wl,
+                                                 v4i (&ring)[kRing][COUT / 32],
+                                                 const int (&ci)[3], int h,
+                                                 f32x16 (&acc)[COUT / 32][3]) {
   using G = Geo<P>;
   constexpr int NT = COUT / 32;
   constexpr int KC = CIN / G::KSTEP;
@@ -155,46 +193,48 @@ __device__ __forceinline__ void conv3_accumulate(const unsigned char *smem,
   constexpr int D = kRing;
   static_assert(U % D == 0, "ring depth must divide the k-steps of a kernel row");
 
-  v4i ring[D][NT];
+  // LDS address of logical record offset `o` at tap (j, kx): pb + (x ^ o), x = lane-half ^ swizzle
+  int pb[3][3], xo[3][3];
+  auto set_row = [&](int ky) {
 #pragma unroll
-  for (int d = 0; d < D; ++d)
+    for (int j = 0; j < 3; ++j)
 #pragma unroll
-    for (int t = 0; t < NT; ++t) ring[d][t] = wl[(d * NT + t) * 64];
-
-  auto tap_base = [&](int j, int ky, int kx) {
-    const int pp = ci[j] + (ky - 1) * kPitch + (kx - 1);
-    return pp * G::PIXB + (((h ^ (pp >> 2)) & 1) << 4);
+      for (int kx = 0; kx < 3; ++kx) {
+        const int pos = ci[j] + (ky - 1) * kPitch + (kx - 1);
+        pb[j][kx] = pos * G::PIXB;
+        xo[j][kx] = (h << 4) ^ swz_of<P>(pos);
+      }
   };
-  int base[3][3];
-#pragma unroll
-  for (int j = 0; j < 3; ++j)
-#pragma unroll
-    for (int kx = 0; kx < 3; ++kx) base[j][kx] = tap_base(j, 0, kx);
+  auto frag_at = [&](int j, int kx, int o) {
+    if constexpr (G::PADDED) {
+      return *reinterpret_cast<const v4i *>(smem + pb[j][kx] + xo[j][kx] + o);
+    } else {
+      return *reinterpret_cast<const v4i *>(smem + pb[j][kx] + (xo[j][kx] ^ o));
+    }
+  };
+  set_row(0);
   v4i bcur[3], lcur[3];
 #pragma unroll
   for (int j = 0; j < 3; ++j) {
-    bcur[j] = *reinterpret_cast<const v4i *>(smem + base[j][0]);
-    if constexpr (P::SPLIT) lcur[j] = *reinterpret_cast<const v4i *>(smem + base[j][0] + G::PLANE);
+    bcur[j] = frag_at(j, 0, 0);
+    if constexpr (P::SPLIT) lcur[j] = frag_at(j, 0, G::PLANE);
   }
 
 #pragma unroll 1
   for (int ky = 0; ky < 3; ++ky) {
-    int nbase[3][3];  // next kernel row (wraps to row 0 after the last: one harmless extra fetch)
-    const int kyn = ky == 2 ? 0 : ky + 1;
-#pragma unroll
-    for (int j = 0; j < 3; ++j)
-#pragma unroll
-      for (int kx = 0; kx < 3; ++kx) nbase[j][kx] = tap_base(j, kyn, kx);
     const v4i *wn = wl + (size_t)(ky * U + D) * NT * 64;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       // fetch the activation fragments of the next k-step while this step's MFMAs run
+      // (after the last tap this wraps to kernel row 0: one harmless extra fetch)
+      if (u + 1 == U) set_row(ky == 2 ? 0 : ky + 1);
+      const int kxn = (u + 1 < U) ? (u + 1) / KC : 0;
+      const int on = (u + 1 < U) ? ((u + 1) % KC) * 32 : 0;
       v4i bnext[3], lnext[3];
 #pragma unroll
       for (int j = 0; j < 3; ++j) {
-        const int a = (u + 1 < U) ? base[j][(u + 1) / KC] + ((u + 1) % KC) * 32 : nbase[j][0];
-        bnext[j] = *reinterpret_cast<const v4i *>(smem + a);
-        if constexpr (P::SPLIT) lnext[j] = *reinterpret_cast<const v4i *>(smem + a + G::PLANE);
+        bnext[j] = frag_at(j, kxn, on);
+        if constexpr (P::SPLIT) lnext[j] = frag_at(j, kxn, on + G::PLANE);
       }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -217,10 +257,6 @@ __device__ __forceinline__ void conv3_accumulate(const unsigned char *smem,
         if constexpr (P::SPLIT) lcur[j] = lnext[j];
       }
     }
-#pragma unroll
-    for (int j = 0; j < 3; ++j)
-#pragma unroll
-      for (int kx = 0; kx < 3; ++kx) base[j][kx] = nbase[j][kx];
   }
 }
 
@@ -234,8 +270,12 @@ __device__ __forceinline__ void store_activations(unsigned char *smem, const int
   constexpr int NT = COUT / 32;
 #pragma unroll
   for (int j = 0; j < 3; ++j) {
-    const int pbase = ci[j] * G::PIXB;
-    const int swz = ((ci[j] >> 2) & 1) << 4;
+    // Recompute the lane's store addresses here, every time: hoisted out of the board loop
+    // they would occupy ~100 registers for the whole kernel and end up in scratch memory.
+    int pos = ci[j];
+    asm volatile("" : "+v"(pos));
+    const int pbase = pos * G::PIXB;
+    const int sw = swz_of<P>(pos);
 #pragma unroll
     for (int t = 0; t < NT; ++t)
 #pragma unroll
@@ -244,7 +284,7 @@ __device__ __forceinline__ void store_activations(unsigned char *smem, const int
         float v[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[e] = silu<P>(acc[t][j][4 * q + e]);
-        store4<P>(smem + pbase + ((ch0 * G::EB) ^ swz), v);
+        store4<P>(smem, pbase, sw, ch0 * G::EB, v);
       }
   }
 }
@@ -252,11 +292,13 @@ __device__ __forceinline__ void store_activations(unsigned char *smem, const int
 // accumulators start at the layer's bias: lane (h) register i holds channel 32t + 8(i/4) + 4h + i%4
 template <int N>
 __device__ __forceinline__ void init_acc(f32x16 (&acc)[N][3], const float *__restrict__ bias, int h) {
+  const float *bl = bias + 4 * h;  // one per-lane base; every load below is base + constant
+  asm volatile("" : "+v"(bl));
 #pragma unroll
   for (int t = 0; t < N; ++t)
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      const f32x4 b4 = *reinterpret_cast<const f32x4 *>(bias + 32 * t + 8 * q + 4 * h);
+      const f32x4 b4 = *reinterpret_cast<const f32x4 *>(bl + 32 * t + 8 * q);
 #pragma unroll
       for (int j = 0; j < 3; ++j)
 #pragma unroll
@@ -264,15 +306,19 @@ __device__ __forceinline__ void init_acc(f32x16 (&acc)[N][3], const float *__res
     }
 }
 
-template <class P, int L, int CIN, int COUT>
+// one 3x3 layer that is not the last: accumulate, hand over the next layer's ring, SiLU, store
+template <class P, int L, int NTN>
 __device__ __forceinline__ void mid_layer(unsigned char *smem, const unsigned char *packed,
-                                          const float *tail, const int (&ci)[3],
-                                          const bool (&valid)[3], int h, int lane) {
-  using G = Geo<P>;
+                                          const float *tail,
+                                          v4i (&ring)[kRing][kCoutArr[L] / 32],
+                                          v4i (&next)[kRing][NTN], const int (&ci)[3], int h,
+                                          int lane) {
+  constexpr int CIN = kCinArr[L], COUT = kCoutArr[L];
+  static_assert(NTN == kCoutArr[L + 1] / 32, "ring shape of the following layer");
   f32x16 acc[COUT / 32][3];
   init_acc(acc, tail + bias_offset(L), h);
-  const v4i *wl = reinterpret_cast<const v4i *>(packed + (size_t)G::frag_offset(L) * 1024) + lane;
-  conv3_accumulate<P, CIN, COUT>(smem, wl, ci, h, acc);
+  conv3_accumulate<P, CIN, COUT>(smem, layer_weights<P, L>(packed, lane), ring, ci, h, acc);
+  preload_ring(next, layer_weights<P, L + 1>(packed, lane));
   __syncthreads();  // every wave has finished reading the previous layer
   store_activations<P, COUT>(smem, ci, h, acc);
   __syncthreads();
@@ -311,53 +357,83 @@ __global__ __launch_bounds__(kThreads) void fused_forward_kernel(const FwdParams
   float *lgt = reinterpret_cast<float *>(smem + G::LGT_OFF);
   float *red = reinterpret_cast<float *>(smem + G::RED_OFF);
 
-  for (long long b = blockIdx.x; b < prm.total_boards; b += gridDim.x) {
-    const long long g = b / prm.boards_per_group;
-    const unsigned char *packed = prm.packed + (size_t)g * prm.packed_stride;
+  auto packed_of = [&](long long b) {
+    return prm.packed + (size_t)(b / prm.boards_per_group) * prm.packed_stride;
+  };
+  // input of one board: each thread owns pixels tid and tid+256 (three planes + occupancy)
+  float xin[2][3];
+  unsigned char occin[2];
+  auto fetch_board = [&](long long b) {
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+      const int p = tid + r * kThreads;
+      if (p < kPix) {
+#pragma unroll
+        for (int ch = 0; ch < 3; ++ch)
+          xin[r][ch] = load_x(prm.x, prm.x_dtype, ((size_t)b * 3 + ch) * kPix + p);
+        occin[r] = prm.mask_mode == C6_MASK_LEGAL ? (prm.legal[(size_t)b * kPix + p] == 0) : 0;
+      }
+    }
+  };
+
+  long long b = blockIdx.x;
+  if (b >= prm.total_boards) return;
+  v4i r1[L1Pipe<P>::D][1];
+  preload_ring(r1, layer_weights<P, 0>(packed_of(b), lane));
+  fetch_board(b);
+
+  for (; b < prm.total_boards; b += gridDim.x) {
+    int tidv = tid;  // opaque per board: keeps per-thread staging addresses out of long-lived registers
+    asm volatile("" : "+v"(tidv));
+    const unsigned char *packed = packed_of(b);
     const float *tail = reinterpret_cast<const float *>(packed + G::TAIL_OFF);
 
     __syncthreads();  // previous board fully written out; LDS is free
     // ---- stage the input: zero the shifted copies, then scatter the board ----
     {
       const v4i z = {0, 0, 0, 0};
-      for (int i = tid * 16; i < G::COPIES_BYTES; i += kThreads * 16)
+      for (int i = tidv * 16; i < G::COPIES_BYTES; i += kThreads * 16)
         *reinterpret_cast<v4i *>(smem + i) = z;
     }
     __syncthreads();
-    for (int p = tid; p < kPix; p += kThreads) {
-      const int r = p / kBoard, c = p - r * kBoard;
-      float v[3];
 #pragma unroll
-      for (int ch = 0; ch < 3; ++ch) v[ch] = load_x(prm.x, prm.x_dtype, ((size_t)b * 3 + ch) * kPix + p);
-      unsigned char o = (v[0] != 0.0f) || (v[1] != 0.0f);
-      if (prm.mask_mode == C6_MASK_LEGAL) o = prm.legal[(size_t)b * kPix + p] == 0;
-      if (prm.mask_mode == C6_MASK_NONE) o = 0;
-      occ[p] = o;
+    for (int r = 0; r < 2; ++r) {
+      const int p = tidv + r * kThreads;
+      if (p < kPix) {
+        const int row = p / kBoard, c = p - row * kBoard;
+        unsigned char o = occin[r];
+        if (prm.mask_mode == C6_MASK_INPUT) o = (xin[r][0] != 0.0f) || (xin[r][1] != 0.0f);
+        occ[p] = o;
 #pragma unroll
-      for (int ch = 0; ch < 3; ++ch) {
-        const int row = (r + kK1 / 2) * 3 + ch;
+        for (int ch = 0; ch < 3; ++ch) {
+          const int hrow = (row + kK1 / 2) * 3 + ch;
 #pragma unroll
-        for (int s = 0; s < G::E; ++s) {
-          const int a = s * G::COPY_BYTES + (row * kL1RowPitch + (c + kK1 / 2 - s)) * G::EB;
-          if constexpr (G::EB == 4) {
-            *reinterpret_cast<float *>(smem + a) = v[ch];
-          } else {
-            *reinterpret_cast<unsigned short *>(smem + a) = bits16<P>(v[ch]);
+          for (int s = 0; s < G::E; ++s) {
+            const int a = s * G::COPY_BYTES + (hrow * kL1RowPitch + (c + kK1 / 2 - s)) * G::EB;
+            if constexpr (G::EB == 4) {
+              *reinterpret_cast<float *>(smem + a) = xin[r][ch];
+            } else {
+              *reinterpret_cast<unsigned short *>(smem + a) = bits16<P>(xin[r][ch]);
+            }
           }
         }
       }
     }
+    const long long bn = b + gridDim.x;
+    if (bn < prm.total_boards) fetch_board(bn);  // lands while this board is computed
     __syncthreads();
 
+    v4i r2[kRing][1], r3[kRing][2], r4[kRing][2], r5[kRing][2], r6[kRing][3], r7[kRing][3],
+        r8[kRing][3];
     // ---- layer 1 ----
     {
       f32x16 acc[1][3];
       init_acc(acc, tail + bias_offset(0), h);
-      const v4i *wl = reinterpret_cast<const v4i *>(packed) + lane;
-      conv1_accumulate<P>(smem, wl, l1base, acc);
+      conv1_accumulate<P>(smem, layer_weights<P, 0>(packed, lane), r1, l1base, acc);
+      preload_ring(r2, layer_weights<P, 1>(packed, lane));
       __syncthreads();
       // the copies overlapped the activation tile: restore its zero padding
-      for (int i = tid; i < 60 * (G::PIXB / 16); i += kThreads) {
+      for (int i = tidv; i < 60 * (G::PIXB / 16); i += kThreads) {
         const int k = i / (G::PIXB / 16), w16 = i - k * (G::PIXB / 16);
         // pad positions: 0..19 (top row), 400..420 (bottom row + tail), 20*R (left column)
         const int pos = k < 20 ? k : (k < 41 ? 400 + (k - 20) : (k - 40) * kPitch);
@@ -367,30 +443,31 @@ __global__ __launch_bounds__(kThreads) void fused_forward_kernel(const FwdParams
       store_activations<P, 32>(smem, ci, h, acc);
       __syncthreads();
     }
-    mid_layer<P, 1, 32, 32>(smem, packed, tail, ci, valid, h, lane);
-    mid_layer<P, 2, 32, 64>(smem, packed, tail, ci, valid, h, lane);
-    mid_layer<P, 3, 64, 64>(smem, packed, tail, ci, valid, h, lane);
-    mid_layer<P, 4, 64, 64>(smem, packed, tail, ci, valid, h, lane);
-    mid_layer<P, 5, 64, 96>(smem, packed, tail, ci, valid, h, lane);
-    mid_layer<P, 6, 96, 96>(smem, packed, tail, ci, valid, h, lane);
+    mid_layer<P, 1, 2>(smem, packed, tail, r2, r3, ci, h, lane);
+    mid_layer<P, 2, 2>(smem, packed, tail, r3, r4, ci, h, lane);
+    mid_layer<P, 3, 2>(smem, packed, tail, r4, r5, ci, h, lane);
+    mid_layer<P, 4, 3>(smem, packed, tail, r5, r6, ci, h, lane);
+    mid_layer<P, 5, 3>(smem, packed, tail, r6, r7, ci, h, lane);
+    mid_layer<P, 6, 3>(smem, packed, tail, r7, r8, ci, h, lane);
 
     // ---- layer 8 + both 1x1 heads straight from the fp32 accumulators ----
     {
       f32x16 acc[3][3];
       init_acc(acc, tail + bias_offset(7), h);
-      const v4i *wl = reinterpret_cast<const v4i *>(packed + (size_t)G::frag_offset(7) * 1024) + lane;
-      conv3_accumulate<P, 96, 96>(smem, wl, ci, h, acc);
+      conv3_accumulate<P, 96, 96>(smem, layer_weights<P, 7>(packed, lane), r8, ci, h, acc);
+      if (bn < prm.total_boards) preload_ring(r1, layer_weights<P, 0>(packed_of(bn), lane));
       const float *polw = tail + kBiasTotal;
       const float *valw = polw + kHeadC;
+      const float *pwl = polw + 4 * h;  // per-lane base: channel 32t + 8q + 4h + e
+      asm volatile("" : "+v"(pwl));
       float pol[3] = {0.0f, 0.0f, 0.0f};
       float vsum = 0.0f;
 #pragma unroll
       for (int t = 0; t < 3; ++t)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const int ch0 = 32 * t + 8 * q + 4 * h;
-          const f32x4 pw = *reinterpret_cast<const f32x4 *>(polw + ch0);
-          const f32x4 vw = *reinterpret_cast<const f32x4 *>(valw + ch0);
+          const f32x4 pw = *reinterpret_cast<const f32x4 *>(pwl + 32 * t + 8 * q);
+          const f32x4 vw = *reinterpret_cast<const f32x4 *>(pwl + kHeadC + 32 * t + 8 * q);
 #pragma unroll
           for (int j = 0; j < 3; ++j)
 #pragma unroll
