@@ -37,6 +37,8 @@ def main() -> int:
     ap.add_argument("--precision", default=HEADLINE, choices=["bf16x2", "bf16", "fp16", "fp32"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="headline + roofline only")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch one plain 256 MiB device copy (reference for rocprof byte counters)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: the forward shards by board with no exchange step, "
@@ -75,6 +77,12 @@ def main() -> int:
             wall = (time.perf_counter() - t0) / steps
         kernel = sum(a.elapsed_time(b) for a, b in evs) / steps * 1e-3
         return wall, kernel
+
+    if args.calibrate_copy:
+        src = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device=dev)   # 256 MiB
+        dst = src + 1.0          # one elementwise kernel: reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
 
     wall, kern = run_mode(args.precision, K, W)
     value = B / wall
