@@ -98,6 +98,11 @@ int c6_forward(const void *x, int x_dtype, int64_t groups, int64_t boards_per_gr
     return C6_EINVAL;
   }
   if (boards_per_group == 0) return C6_OK;  // empty batch: nothing to do
+  if (groups > 0x7fffffffLL / boards_per_group) {
+    set_error("c6_forward: %lld x %lld boards exceed the 2^31-1 boards one launch can index",
+              (long long)groups, (long long)boards_per_group);
+    return C6_EINVAL;
+  }
   if (x == nullptr || packed == nullptr) {
     set_error("c6_forward: x and packed must not be null");
     return C6_EINVAL;

@@ -17,6 +17,18 @@
 
 namespace c6 {
 
+// Optional phase timestamps for kernel tuning (never compiled into the shipped library).
+#ifdef C6_TRACE
+__device__ long long g_trace[256 * 4 * 64];
+#define C6_MARK(idx)                                                                       \
+  do {                                                                                     \
+    if (trace_on && lane == 0 && blockIdx.x < 256)                                         \
+      g_trace[(blockIdx.x * 4 + wave) * 64 + (idx)] = (long long)__builtin_readcyclecounter(); \
+  } while (0)
+#else
+#define C6_MARK(idx) do { } while (0)
+#endif
+
 // ------------------------------------------------------------------------
 // precision-specific primitives
 // ------------------------------------------------------------------------
@@ -73,24 +85,40 @@ template <class P> __device__ __forceinline__ int swz_of(int pos) {
   }
 }
 
-// store four consecutive channels (logical byte offset `o` inside the record) of position `pos`
-template <class P>
-__device__ __forceinline__ void store4(unsigned char *smem, int pbase, int sw, int o,
-                                       const float (&v)[4]) {
+// four consecutive channels of one position, converted to the storage type
+template <class P> struct Packed4 {
+  v2i hi;  // 16-bit modes: 4 values; split mode: the leading bf16 parts
+  v2i lo;  // split mode only: what the first rounding dropped
+};
+template <> struct Packed4<PrecF32> {
+  f32x4 v;
+};
+
+template <class P> __device__ __forceinline__ Packed4<P> pack4(const float (&v)[4]) {
+  Packed4<P> r;
   if constexpr (P::EB == 4) {
-    const f32x4 w = {v[0], v[1], v[2], v[3]};
-    *reinterpret_cast<f32x4 *>(smem + pbase + (o ^ sw)) = w;
+    r.v = f32x4{v[0], v[1], v[2], v[3]};
   } else {
-    v2i w;
-    w[0] = pack2<P>(v[0], v[1]);
-    w[1] = pack2<P>(v[2], v[3]);
-    *reinterpret_cast<v2i *>(smem + pbase + (o ^ sw)) = w;
-    if constexpr (P::SPLIT) {  // low-order part: what the first rounding dropped
-      v2i q;
-      q[0] = pack2<P>(v[0] - bf16_lo(w[0]), v[1] - bf16_hi(w[0]));
-      q[1] = pack2<P>(v[2] - bf16_lo(w[1]), v[3] - bf16_hi(w[1]));
-      *reinterpret_cast<v2i *>(smem + pbase + ((o + Geo<P>::PLANE) ^ sw)) = q;
+    r.hi[0] = pack2<P>(v[0], v[1]);
+    r.hi[1] = pack2<P>(v[2], v[3]);
+    if constexpr (P::SPLIT) {
+      r.lo[0] = pack2<P>(v[0] - bf16_lo(r.hi[0]), v[1] - bf16_hi(r.hi[0]));
+      r.lo[1] = pack2<P>(v[2] - bf16_lo(r.hi[1]), v[3] - bf16_hi(r.hi[1]));
     }
+  }
+  return r;
+}
+
+// store at logical byte offset `o` inside the record of the position at `pbase` (swizzle `sw`)
+template <class P>
+__device__ __forceinline__ void put4(unsigned char *smem, int pbase, int sw, int o,
+                                     const Packed4<P> &r) {
+  if constexpr (P::EB == 4) {
+    *reinterpret_cast<f32x4 *>(smem + pbase + (o ^ sw)) = r.v;
+  } else {
+    *reinterpret_cast<v2i *>(smem + pbase + (o ^ sw)) = r.hi;
+    if constexpr (P::SPLIT)
+      *reinterpret_cast<v2i *>(smem + pbase + ((o + Geo<P>::PLANE) ^ sw)) = r.lo;
   }
 }
 
@@ -137,55 +165,81 @@ __device__ __forceinline__ const v4i *layer_weights(const unsigned char *packed,
 }
 
 // ------------------------------------------------------------------------
-// first layer: 23x23 on 3 planes, K = (ky, plane, kx24) split over lane halves
+// K-loops.  Each layer runs as two passes over K: pass A accumulates pixel
+// tiles 0 and 1, pass B pixel tile 2.  While pass B's MFMAs run, the same wave
+// applies SiLU to pass A's finished accumulators ("side work"), so two thirds
+// of the epilogue's VALU work hides under matrix-core time.  Pass A's weight
+// prefetch wraps around so that pass B starts with a full ring.
 // ------------------------------------------------------------------------
-template <class P>
-__device__ __forceinline__ void conv1_accumulate(const unsigned char *smem,
-                                                 const v4i *__restrict__ wl,
-                                                 v4i (&ring)[L1Pipe<P>::D][1],
-                                                 const int (&l1base)[3], f32x16 (&acc)[1][3]) {
+// Two-pass K-loops (pixel tiles {0,1} then {2} with the epilogue of the first pass riding
+// along) were measured slower than one pass: the second pass re-streams every weight
+// fragment for a third of the MFMA work and becomes L1-bound.  Kept switchable.
+constexpr bool kTwoPass = false;
+
+// Issue order inside one k-step: memory instructions are dealt out one at a time between
+// MFMAs.  Issued back to back, three ds_read_b128 or global_load_dwordx4 hold the wave's
+// issue port longer than one MFMA executes and the matrix pipe runs dry.
+template <int N_MFMA, int N_DSREAD, int N_VMEM> __device__ __forceinline__ void interleave_step() {
+#pragma unroll
+  for (int i = 0; i < N_MFMA; ++i) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+    if (i < N_DSREAD) {
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+    } else if (i < N_DSREAD + N_VMEM) {
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one global load
+    }
+  }
+}
+
+struct NoSide {
+  __device__ __forceinline__ void operator()(int) const {}
+};
+
+// first layer: 23x23 on 3 planes, K = (ky, plane, kx24) split over lane halves
+template <class P, int J0, int NJ, bool WRAP, bool UNROLL, class Side>
+__device__ __forceinline__ void conv1_pass(const unsigned char *smem, const v4i *__restrict__ wl,
+                                           v4i (&ring)[L1Pipe<P>::D][1], const int (&l1base)[3],
+                                           f32x16 (&acc)[1][3], Side side) {
   using G = Geo<P>;
   using PP = L1Pipe<P>;
-  constexpr int CPR = PP::CPR, U = PP::U, D = PP::D;
+  constexpr int CPR = PP::CPR, U = PP::U, D = PP::D, ITERS = PP::ITERS;
   constexpr int ROWB = kL1RowPitch * G::EB;
 
-  v4i bcur[3];
+  v4i bcur[NJ];
 #pragma unroll
-  for (int j = 0; j < 3; ++j) bcur[j] = *reinterpret_cast<const v4i *>(smem + l1base[j]);
-#pragma unroll 1
-  for (int it = 0; it < PP::ITERS; ++it) {
+  for (int j = 0; j < NJ; ++j) bcur[j] = *reinterpret_cast<const v4i *>(smem + l1base[J0 + j]);
+#pragma unroll(UNROLL ? ITERS : 1)
+  for (int it = 0; it < ITERS; ++it) {
     const int adv = it * PP::ROWS_BODY * ROWB;
-    const v4i *wn = wl + (size_t)(it * U + D) * 64;
+    const v4i *wlo = wl + (size_t)(it * U + D) * 64;
+    const v4i *whi = (WRAP && it == ITERS - 1) ? wl - (size_t)(U - D) * 64 : wlo;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       // operand fragments of the NEXT k-step are fetched while this step's MFMAs run; after
       // the last step this reads the zero row / the next copy, which is harmless
       const int un = u + 1;
       const int offn = (un / CPR) * ROWB + (un % CPR) * 16;
-      v4i bnext[3];
+      v4i bnext[NJ];
 #pragma unroll
-      for (int j = 0; j < 3; ++j)
-        bnext[j] = *reinterpret_cast<const v4i *>(smem + l1base[j] + adv + offn);
+      for (int j = 0; j < NJ; ++j)
+        bnext[j] = *reinterpret_cast<const v4i *>(smem + l1base[J0 + j] + adv + offn);
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) mma<P>(ring[u % D][0], bcur[j], acc[0][J0 + j]);
+      ring[u % D][0] = (u < U - D ? wlo : whi)[u * 64];  // k-step it*U + u + D (wrapped or over-read)
+      side(it * U + u);
+      interleave_step<NJ * (P::EB == 4 ? 4 : 1), NJ, 1>();
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int j = 0; j < 3; ++j) mma<P>(ring[u % D][0], bcur[j], acc[0][j]);
-      ring[u % D][0] = wn[u * 64];  // k-step (it*U + u + D); the tail over-reads the next layer
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int j = 0; j < 3; ++j) bcur[j] = bnext[j];
+      for (int j = 0; j < NJ; ++j) bcur[j] = bnext[j];
     }
   }
 }
 
-// ------------------------------------------------------------------------
 // 3x3 layers: K = (tap, cin), cin fastest; taps are constant position offsets
-// ------------------------------------------------------------------------
-template <class P, int CIN, int COUT>
-__device__ __forceinline__ void conv3_accumulate(const unsigned char *smem,
-                                                 const v4i *__restrict__ wl,
-                                                 v4i (&ring)[kRing][COUT / 32],
-                                                 const int (&ci)[3], int h,
-                                                 f32x16 (&acc)[COUT / 32][3]) {
+template <class P, int CIN, int COUT, int J0, int NJ, bool WRAP, bool UNROLL, class Side>
+__device__ __forceinline__ void conv3_pass(const unsigned char *smem, const v4i *__restrict__ wl,
+                                           v4i (&ring)[kRing][COUT / 32], const int (&ci)[3],
+                                           int h, f32x16 (&acc)[COUT / 32][3], Side side) {
   using G = Geo<P>;
   constexpr int NT = COUT / 32;
   constexpr int KC = CIN / G::KSTEP;
@@ -194,13 +248,13 @@ __device__ __forceinline__ void conv3_accumulate(const unsigned char *smem,
   static_assert(U % D == 0, "ring depth must divide the k-steps of a kernel row");
 
   // LDS address of logical record offset `o` at tap (j, kx): pb + (x ^ o), x = lane-half ^ swizzle
-  int pb[3][3], xo[3][3];
+  int pb[NJ][3], xo[NJ][3];
   auto set_row = [&](int ky) {
 #pragma unroll
-    for (int j = 0; j < 3; ++j)
+    for (int j = 0; j < NJ; ++j)
 #pragma unroll
       for (int kx = 0; kx < 3; ++kx) {
-        const int pos = ci[j] + (ky - 1) * kPitch + (kx - 1);
+        const int pos = ci[J0 + j] + (ky - 1) * kPitch + (kx - 1);
         pb[j][kx] = pos * G::PIXB;
         xo[j][kx] = (h << 4) ^ swz_of<P>(pos);
       }
@@ -213,16 +267,17 @@ __device__ __forceinline__ void conv3_accumulate(const unsigned char *smem,
     }
   };
   set_row(0);
-  v4i bcur[3], lcur[3];
+  v4i bcur[NJ], lcur[NJ];
 #pragma unroll
-  for (int j = 0; j < 3; ++j) {
+  for (int j = 0; j < NJ; ++j) {
     bcur[j] = frag_at(j, 0, 0);
     if constexpr (P::SPLIT) lcur[j] = frag_at(j, 0, G::PLANE);
   }
 
-#pragma unroll 1
+#pragma unroll(UNROLL ? 3 : 1)
   for (int ky = 0; ky < 3; ++ky) {
-    const v4i *wn = wl + (size_t)(ky * U + D) * NT * 64;
+    const v4i *wlo = wl + (size_t)(ky * U + D) * NT * 64;
+    const v4i *whi = (WRAP && ky == 2) ? wl - (size_t)(U - D) * NT * 64 : wlo;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       // fetch the activation fragments of the next k-step while this step's MFMAs run
@@ -230,29 +285,39 @@ __device__ __forceinline__ void conv3_accumulate(const unsigned char *smem,
       if (u + 1 == U) set_row(ky == 2 ? 0 : ky + 1);
       const int kxn = (u + 1 < U) ? (u + 1) / KC : 0;
       const int on = (u + 1 < U) ? ((u + 1) % KC) * 32 : 0;
-      v4i bnext[3], lnext[3];
+      v4i bnext[NJ], lnext[NJ];
 #pragma unroll
-      for (int j = 0; j < 3; ++j) {
+      for (int j = 0; j < NJ; ++j) {
         bnext[j] = frag_at(j, kxn, on);
         if constexpr (P::SPLIT) lnext[j] = frag_at(j, kxn, on + G::PLANE);
       }
-      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int t = 0; t < NT; ++t)
 #pragma unroll
-        for (int j = 0; j < 3; ++j) mma<P>(ring[u % D][t], bcur[j], acc[t][j]);
+        for (int j = 0; j < NJ; ++j) mma<P>(ring[u % D][t], bcur[j], acc[t][J0 + j]);
       if constexpr (P::SPLIT) {
 #pragma unroll
         for (int t = 0; t < NT; ++t)
 #pragma unroll
-          for (int j = 0; j < 3; ++j) mma<P>(ring[u % D][t], lcur[j], acc[t][j]);
+          for (int j = 0; j < NJ; ++j) mma<P>(ring[u % D][t], lcur[j], acc[t][J0 + j]);
       }
-      // weights of k-step u+D replace the ones just consumed (the tail over-reads the next layer)
+      // weights of k-step u+D (wrapped to the layer start, or over-reading into the next layer)
+#if defined(C6_EXP_FEWLOADS)   // tuning experiment only: a third of the weight traffic (wrong results)
+      ring[u % D][0] = (u < U - D ? wlo : whi)[(u * NT) * 64];
 #pragma unroll
-      for (int t = 0; t < NT; ++t) ring[u % D][t] = wn[(u * NT + t) * 64];
+      for (int t = 1; t < NT; ++t) ring[u % D][t] = ring[u % D][0];
+#elif defined(C6_EXP_SAMEADDR)  // tuning experiment only: every load hits the same lines (wrong results)
+#pragma unroll
+      for (int t = 0; t < NT; ++t) ring[u % D][t] = wl[t * 64 + (u & 1) * 4096];
+#else
+#pragma unroll
+      for (int t = 0; t < NT; ++t) ring[u % D][t] = (u < U - D ? wlo : whi)[(u * NT + t) * 64];
+#endif
+      side(ky * U + u);
+      interleave_step<NT * NJ * (P::SPLIT ? 2 : 1) * (P::EB == 4 ? 4 : 1), NJ * (P::SPLIT ? 2 : 1), NT>();
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int j = 0; j < 3; ++j) {
+      for (int j = 0; j < NJ; ++j) {
         bcur[j] = bnext[j];
         if constexpr (P::SPLIT) lcur[j] = lnext[j];
       }
@@ -260,33 +325,30 @@ __device__ __forceinline__ void conv3_accumulate(const unsigned char *smem,
   }
 }
 
-// SiLU + store of one layer's accumulators (bias already added at init) into the
-// activation tile.  Lanes beyond pixel 360 shadow pixel 360 (same inputs, same
-// results, same address), so every lane stores unconditionally.
-template <class P, int COUT>
-__device__ __forceinline__ void store_activations(unsigned char *smem, const int (&ci)[3], int h,
-                                                  const f32x16 (&acc)[COUT / 32][3]) {
+// SiLU of the four accumulators (tile t, pixel tile j, quad q): bias was added at init
+template <class P, int NT>
+__device__ __forceinline__ Packed4<P> silu_quad(const f32x16 (&acc)[NT][3], int t, int j, int q) {
+  float v[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) v[e] = silu<P>(acc[t][j][4 * q + e]);
+  return pack4<P>(v);
+}
+
+// Write one pixel tile's packed activations.  Lanes beyond pixel 360 shadow pixel 360 (same
+// inputs, same results, same address), so every lane stores unconditionally.  The lane's
+// addresses are recomputed here every time: hoisted out of the board loop they would occupy
+// ~100 registers for the whole kernel and end up in scratch memory.
+template <class P, int NT, class Get>
+__device__ __forceinline__ void store_tile(unsigned char *smem, int pos_in, int h, Get get) {
   using G = Geo<P>;
-  constexpr int NT = COUT / 32;
+  int pos = pos_in;
+  asm volatile("" : "+v"(pos));
+  const int pbase = pos * G::PIXB;
+  const int sw = swz_of<P>(pos);
 #pragma unroll
-  for (int j = 0; j < 3; ++j) {
-    // Recompute the lane's store addresses here, every time: hoisted out of the board loop
-    // they would occupy ~100 registers for the whole kernel and end up in scratch memory.
-    int pos = ci[j];
-    asm volatile("" : "+v"(pos));
-    const int pbase = pos * G::PIXB;
-    const int sw = swz_of<P>(pos);
+  for (int t = 0; t < NT; ++t)
 #pragma unroll
-    for (int t = 0; t < NT; ++t)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int ch0 = 32 * t + 8 * q + 4 * h;
-        float v[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = silu<P>(acc[t][j][4 * q + e]);
-        store4<P>(smem, pbase, sw, ch0 * G::EB, v);
-      }
-  }
+    for (int q = 0; q < 4; ++q) put4<P>(smem, pbase, sw, (32 * t + 8 * q + 4 * h) * G::EB, get(t, q));
 }
 
 // accumulators start at the layer's bias: lane (h) register i holds channel 32t + 8(i/4) + 4h + i%4
@@ -306,22 +368,70 @@ __device__ __forceinline__ void init_acc(f32x16 (&acc)[N][3], const float *__res
     }
 }
 
-// one 3x3 layer that is not the last: accumulate, hand over the next layer's ring, SiLU, store
+// barrier; pass A's packed activations and pass B's (SiLU here) go to the tile; barrier
+template <class P, int NT, class Pre>
+__device__ __forceinline__ void finish_layer(unsigned char *smem, const int (&ci)[3], int h,
+                                             const f32x16 (&acc)[NT][3],
+                                             const Packed4<P> (&pk)[2][NT][4], Pre before_store) {
+  __syncthreads();  // every wave has finished reading the layer's input
+  before_store();
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    if constexpr (kTwoPass) {
+      store_tile<P, NT>(smem, ci[j], h, [&](int t, int q) { return pk[j][t][q]; });
+    } else {
+      store_tile<P, NT>(smem, ci[j], h, [&](int t, int q) { return silu_quad<P, NT>(acc, t, j, q); });
+    }
+  }
+  store_tile<P, NT>(smem, ci[2], h, [&](int t, int q) { return silu_quad<P, NT>(acc, t, 2, q); });
+  __syncthreads();
+}
+
+// side work of pass B: SiLU + pack of pass A's accumulators, one quad per k-step
+template <class P, int NT> struct SiluSide {
+  const f32x16 (&acc)[NT][3];
+  Packed4<P> (&pk)[2][NT][4];
+  __device__ __forceinline__ void operator()(int step) const {
+    if (step < 8 * NT) {
+      const int j = step / (4 * NT), t = (step / 4) % NT, q = step % 4;
+      pk[j][t][q] = silu_quad<P, NT>(acc, t, j, q);
+    }
+  }
+};
+
+// one 3x3 layer that is not the last
 template <class P, int L, int NTN>
 __device__ __forceinline__ void mid_layer(unsigned char *smem, const unsigned char *packed,
                                           const float *tail,
                                           v4i (&ring)[kRing][kCoutArr[L] / 32],
                                           v4i (&next)[kRing][NTN], const int (&ci)[3], int h,
-                                          int lane) {
-  constexpr int CIN = kCinArr[L], COUT = kCoutArr[L];
+                                          int lane, bool trace_on = false) {
+  constexpr int CIN = kCinArr[L], COUT = kCoutArr[L], NT = COUT / 32;
   static_assert(NTN == kCoutArr[L + 1] / 32, "ring shape of the following layer");
-  f32x16 acc[COUT / 32][3];
+  f32x16 acc[NT][3];
+  Packed4<P> pk[2][NT][4];
   init_acc(acc, tail + bias_offset(L), h);
-  conv3_accumulate<P, CIN, COUT>(smem, layer_weights<P, L>(packed, lane), ring, ci, h, acc);
+  const v4i *wl = layer_weights<P, L>(packed, lane);
+  if constexpr (kTwoPass) {
+    conv3_pass<P, CIN, COUT, 0, 2, true, false>(smem, wl, ring, ci, h, acc, NoSide{});
+    conv3_pass<P, CIN, COUT, 2, 1, false, true>(smem, wl, ring, ci, h, acc, SiluSide<P, NT>{acc, pk});
+  } else {
+    conv3_pass<P, CIN, COUT, 0, 3, false, false>(smem, wl, ring, ci, h, acc, NoSide{});
+  }
   preload_ring(next, layer_weights<P, L + 1>(packed, lane));
-  __syncthreads();  // every wave has finished reading the previous layer
-  store_activations<P, COUT>(smem, ci, h, acc);
-  __syncthreads();
+#ifdef C6_TRACE
+  {
+    const int wave = threadIdx.x >> 6;
+    C6_MARK(4 + 2 * L);
+  }
+#endif
+  finish_layer<P, NT>(smem, ci, h, acc, pk, [] {});
+#ifdef C6_TRACE
+  {
+    const int wave = threadIdx.x >> 6;
+    C6_MARK(5 + 2 * L);
+  }
+#endif
 }
 
 // ------------------------------------------------------------------------
@@ -357,8 +467,9 @@ __global__ __launch_bounds__(kThreads) void fused_forward_kernel(const FwdParams
   float *lgt = reinterpret_cast<float *>(smem + G::LGT_OFF);
   float *red = reinterpret_cast<float *>(smem + G::RED_OFF);
 
+  const unsigned per_group = (unsigned)prm.boards_per_group;  // board counts fit 32 bits (host-checked)
   auto packed_of = [&](long long b) {
-    return prm.packed + (size_t)(b / prm.boards_per_group) * prm.packed_stride;
+    return prm.packed + (size_t)((unsigned)b / per_group) * prm.packed_stride;
   };
   // input of one board: each thread owns pixels tid and tid+256 (three planes + occupancy)
   float xin[2][3];
@@ -388,7 +499,14 @@ __global__ __launch_bounds__(kThreads) void fused_forward_kernel(const FwdParams
     const unsigned char *packed = packed_of(b);
     const float *tail = reinterpret_cast<const float *>(packed + G::TAIL_OFF);
 
+#ifdef C6_TRACE
+    const bool trace_on = (b == blockIdx.x + 2LL * gridDim.x);  // third board of this workgroup
+#else
+    const bool trace_on = false;
+    (void)trace_on;
+#endif
     __syncthreads();  // previous board fully written out; LDS is free
+    C6_MARK(0);
     // ---- stage the input: zero the shifted copies, then scatter the board ----
     {
       const v4i z = {0, 0, 0, 0};
@@ -422,62 +540,87 @@ __global__ __launch_bounds__(kThreads) void fused_forward_kernel(const FwdParams
     const long long bn = b + gridDim.x;
     if (bn < prm.total_boards) fetch_board(bn);  // lands while this board is computed
     __syncthreads();
+    C6_MARK(1);
 
     v4i r2[kRing][1], r3[kRing][2], r4[kRing][2], r5[kRing][2], r6[kRing][3], r7[kRing][3],
         r8[kRing][3];
     // ---- layer 1 ----
     {
       f32x16 acc[1][3];
+      Packed4<P> pk[2][1][4];
       init_acc(acc, tail + bias_offset(0), h);
-      conv1_accumulate<P>(smem, layer_weights<P, 0>(packed, lane), r1, l1base, acc);
-      preload_ring(r2, layer_weights<P, 1>(packed, lane));
-      __syncthreads();
-      // the copies overlapped the activation tile: restore its zero padding
-      for (int i = tidv; i < 60 * (G::PIXB / 16); i += kThreads) {
-        const int k = i / (G::PIXB / 16), w16 = i - k * (G::PIXB / 16);
-        // pad positions: 0..19 (top row), 400..420 (bottom row + tail), 20*R (left column)
-        const int pos = k < 20 ? k : (k < 41 ? 400 + (k - 20) : (k - 40) * kPitch);
-        const v4i z = {0, 0, 0, 0};
-        *reinterpret_cast<v4i *>(smem + pos * G::PIXB + w16 * 16) = z;
+      const v4i *wl = layer_weights<P, 0>(packed, lane);
+      if constexpr (kTwoPass) {
+        conv1_pass<P, 0, 2, true, false>(smem, wl, r1, l1base, acc, NoSide{});
+        conv1_pass<P, 2, 1, false, true>(smem, wl, r1, l1base, acc, SiluSide<P, 1>{acc, pk});
+      } else {
+        conv1_pass<P, 0, 3, false, false>(smem, wl, r1, l1base, acc, NoSide{});
       }
-      store_activations<P, 32>(smem, ci, h, acc);
-      __syncthreads();
+      preload_ring(r2, layer_weights<P, 1>(packed, lane));
+      C6_MARK(2);
+      finish_layer<P, 1>(smem, ci, h, acc, pk, [&] {
+        // the copies overlapped the activation tile: restore its zero padding
+        for (int i = tidv; i < 60 * (G::PIXB / 16); i += kThreads) {
+          const int k = i / (G::PIXB / 16), w16 = i - k * (G::PIXB / 16);
+          // pad positions: 0..19 (top row), 400..420 (bottom row + tail), 20*R (left column)
+          const int pos = k < 20 ? k : (k < 41 ? 400 + (k - 20) : (k - 40) * kPitch);
+          const v4i z = {0, 0, 0, 0};
+          *reinterpret_cast<v4i *>(smem + pos * G::PIXB + w16 * 16) = z;
+        }
+      });
     }
-    mid_layer<P, 1, 2>(smem, packed, tail, r2, r3, ci, h, lane);
-    mid_layer<P, 2, 2>(smem, packed, tail, r3, r4, ci, h, lane);
-    mid_layer<P, 3, 2>(smem, packed, tail, r4, r5, ci, h, lane);
-    mid_layer<P, 4, 3>(smem, packed, tail, r5, r6, ci, h, lane);
-    mid_layer<P, 5, 3>(smem, packed, tail, r6, r7, ci, h, lane);
-    mid_layer<P, 6, 3>(smem, packed, tail, r7, r8, ci, h, lane);
+    C6_MARK(3);
+    mid_layer<P, 1, 2>(smem, packed, tail, r2, r3, ci, h, lane, trace_on);
+    mid_layer<P, 2, 2>(smem, packed, tail, r3, r4, ci, h, lane, trace_on);
+    mid_layer<P, 3, 2>(smem, packed, tail, r4, r5, ci, h, lane, trace_on);
+    mid_layer<P, 4, 3>(smem, packed, tail, r5, r6, ci, h, lane, trace_on);
+    mid_layer<P, 5, 3>(smem, packed, tail, r6, r7, ci, h, lane, trace_on);
+    mid_layer<P, 6, 3>(smem, packed, tail, r7, r8, ci, h, lane, trace_on);
 
     // ---- layer 8 + both 1x1 heads straight from the fp32 accumulators ----
     {
       f32x16 acc[3][3];
       init_acc(acc, tail + bias_offset(7), h);
-      conv3_accumulate<P, 96, 96>(smem, layer_weights<P, 7>(packed, lane), r8, ci, h, acc);
-      if (bn < prm.total_boards) preload_ring(r1, layer_weights<P, 0>(packed_of(bn), lane));
       const float *polw = tail + kBiasTotal;
       const float *valw = polw + kHeadC;
       const float *pwl = polw + 4 * h;  // per-lane base: channel 32t + 8q + 4h + e
       asm volatile("" : "+v"(pwl));
       float pol[3] = {0.0f, 0.0f, 0.0f};
       float vsum = 0.0f;
+      // heads of pixel tile j, quad (t, q): policy dot and value dot of four channels
+      auto head_quad = [&](int t, int j, int q) {
+        const f32x4 pw = *reinterpret_cast<const f32x4 *>(pwl + 32 * t + 8 * q);
+        const f32x4 vw = *reinterpret_cast<const f32x4 *>(pwl + kHeadC + 32 * t + 8 * q);
+        float vs = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float a = silu<P>(acc[t][j][4 * q + e]);
+          pol[j] = fmaf(a, pw[e], pol[j]);
+          vs = fmaf(a, vw[e], vs);
+        }
+        vsum += valid[j] ? vs : 0.0f;
+      };
+      const v4i *wl = layer_weights<P, 7>(packed, lane);
+      if constexpr (kTwoPass) {
+        conv3_pass<P, 96, 96, 0, 2, true, false>(smem, wl, r8, ci, h, acc, NoSide{});
+        conv3_pass<P, 96, 96, 2, 1, false, true>(smem, wl, r8, ci, h, acc, [&](int step) {
+          if (step < 24) head_quad((step / 4) % 3, step / 12, step % 4);
+        });
+      } else {
+        conv3_pass<P, 96, 96, 0, 3, false, false>(smem, wl, r8, ci, h, acc, NoSide{});
+      }
+      if (bn < prm.total_boards) preload_ring(r1, layer_weights<P, 0>(packed_of(bn), lane));
+      C6_MARK(18);
+#pragma unroll
+      for (int j = 0; j < (kTwoPass ? 0 : 2); ++j)
+#pragma unroll
+        for (int t = 0; t < 3; ++t)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) head_quad(t, j, q);
 #pragma unroll
       for (int t = 0; t < 3; ++t)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const f32x4 pw = *reinterpret_cast<const f32x4 *>(pwl + 32 * t + 8 * q);
-          const f32x4 vw = *reinterpret_cast<const f32x4 *>(pwl + kHeadC + 32 * t + 8 * q);
-#pragma unroll
-          for (int j = 0; j < 3; ++j)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const float a = silu<P>(acc[t][j][4 * q + e]);
-              pol[j] = fmaf(a, pw[e], pol[j]);
-              const float va = a * vw[e];
-              vsum += valid[j] ? va : 0.0f;
-            }
-        }
+        for (int q = 0; q < 4; ++q) head_quad(t, 2, q);
       const float polb = valw[kHeadC], valb = valw[kHeadC + 1];
 #pragma unroll
       for (int j = 0; j < 3; ++j) {
@@ -491,6 +634,7 @@ __global__ __launch_bounds__(kThreads) void fused_forward_kernel(const FwdParams
         const float s = (red[0] + red[1]) + (red[2] + red[3]);
         prm.value[b] = tanhf(s * (1.0f / kPix) + valb);
       }
+      C6_MARK(19);
     }
 
     // ---- write out: masked logits, optional sampled action ----
@@ -512,8 +656,15 @@ __global__ __launch_bounds__(kThreads) void fused_forward_kernel(const FwdParams
         if (prm.logprob != nullptr) prm.logprob[b] = lp;
       }
     }
+    C6_MARK(20);
   }
 }
+
+#ifdef C6_TRACE
+extern "C" int c6_debug_trace(long long *host_out) {
+  return (int)hipMemcpyFromSymbol(host_out, HIP_SYMBOL(g_trace), sizeof(long long) * 256 * 4 * 64);
+}
+#endif
 
 // ------------------------------------------------------------------------
 // weight repack: PyTorch OIHW fp32 -> MFMA fragment order
