@@ -14,7 +14,7 @@ _PKG = Path(__file__).resolve().parent
 _CSRC = _PKG / "csrc"
 _LIBDIR = _PKG / "lib"
 _SO = _LIBDIR / "libconnect6_amd.so"
-_SOURCES = ("c6_forward.hip", "c6_tail.hip", "c6_api.hip")
+_SOURCES = ("c6_forward.hip", "c6_tail.hip", "c6_generic.hip", "c6_api.hip")
 
 # arithmetic modes (include/connect6_amd.h)
 PREC_F32, PREC_BF16, PREC_F16, PREC_BF16X2 = 0, 1, 2, 3
@@ -29,6 +29,8 @@ EXPORTS = (
     "c6_packed_bytes",
     "c6_pack_weights",
     "c6_forward",
+    "c6_generic_workspace_bytes",
+    "c6_forward_generic",
     "c6_mask_logits",
     "c6_softmax_sample",
     "c6_d4_expand",
@@ -85,6 +87,13 @@ def load() -> ctypes.CDLL:
     lib.c6_forward.restype = i32
     lib.c6_forward.argtypes = [vp, i32, i64, i64, vp, ctypes.c_size_t, i32, vp, vp, i32, vp, f32,
                                vp, f32, vp, vp, vp]
+    ip = ctypes.POINTER(ctypes.c_int)
+    lib.c6_generic_workspace_bytes.restype = i32
+    lib.c6_generic_workspace_bytes.argtypes = [i64, i32, i32, ip, ctypes.POINTER(ctypes.c_size_t)]
+    lib.c6_forward_generic.restype = i32
+    lib.c6_forward_generic.argtypes = [vp, i32, i64, i32, i32, ip, ip, ctypes.POINTER(vp),
+                                       ctypes.POINTER(vp), vp, vp, vp, vp, i32, vp,
+                                       ctypes.c_size_t, vp, vp, i32, vp, f32, vp]
     lib.c6_mask_logits.restype = i32
     lib.c6_mask_logits.argtypes = [vp, vp, i32, i64, ctypes.c_uint32, vp, vp]
     lib.c6_softmax_sample.restype = i32

@@ -24,6 +24,13 @@ int launch_sample(const float *, const uint8_t *, const float *, float, long lon
                   float *, hipStream_t);
 int launch_d4_expand(const void *, int, long long, void *, hipStream_t);
 int launch_d4_reduce(const float *, const float *, long long, float *, float *, hipStream_t);
+size_t generic_workspace_bytes(long long batch, int n, int layers, const int *channels);
+int launch_generic(const void *x, int x_dtype, long long batch, int n, int layers,
+                   const int *kernels, const int *channels, const float *const *conv_w,
+                   const float *const *conv_b, const float *pol_w, const float *pol_b,
+                   const float *val_w, const float *val_b, int prec, void *workspace,
+                   float *logits, float *value, int mask_mode, const uint8_t *legal, float fill,
+                   hipStream_t st);
 
 static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 static int elem_bytes(int dt) { return dt == C6_DT_F32 ? 4 : ((dt == C6_DT_BF16 || dt == C6_DT_F16) ? 2 : 0); }
@@ -138,6 +145,72 @@ int c6_forward(const void *x, int x_dtype, int64_t groups, int64_t boards_per_gr
   fp.actions = reinterpret_cast<long long *>(actions);
   fp.logprob = logprob;
   return dispatch_forward(prec, fp, static_cast<hipStream_t>(stream));
+}
+
+static int check_arch(const char *who, int board, int layers, const int *kernels,
+                      const int *channels) {
+  if (board < 1 || layers < 1 || channels == nullptr) {
+    set_error("%s: board=%d layers=%d out of range or null channel list", who, board, layers);
+    return C6_EINVAL;
+  }
+  for (int l = 0; l < layers; ++l) {
+    if (channels[l] < 1 || (kernels && (kernels[l] < 1 || kernels[l] % 2 == 0))) {
+      set_error("%s: layer %d needs a positive channel count and a positive odd kernel", who, l);
+      return C6_EINVAL;
+    }
+  }
+  return C6_OK;
+}
+
+int c6_generic_workspace_bytes(int64_t batch, int board, int layers, const int *channels,
+                               size_t *bytes) {
+  if (batch < 0 || bytes == nullptr) {
+    set_error("c6_generic_workspace_bytes: negative batch or null output");
+    return C6_EINVAL;
+  }
+  const int rc = check_arch("c6_generic_workspace_bytes", board, layers, nullptr, channels);
+  if (rc != C6_OK) return rc;
+  *bytes = generic_workspace_bytes(batch, board, layers, channels);
+  return C6_OK;
+}
+
+int c6_forward_generic(const void *x, int x_dtype, int64_t batch, int board, int layers,
+                       const int *kernels, const int *channels, const float *const *conv_w,
+                       const float *const *conv_b, const float *pol_w, const float *pol_b,
+                       const float *val_w, const float *val_b, int prec, void *workspace,
+                       size_t workspace_bytes, float *logits, float *value, int mask_mode,
+                       const uint8_t *legal, float fill, void *stream) {
+  if (!valid_prec(prec) || elem_bytes(x_dtype) == 0 || batch < 0 || kernels == nullptr) {
+    set_error("c6_forward_generic: bad precision %d, input type %d, batch %lld or null kernels",
+              prec, x_dtype, (long long)batch);
+    return C6_EINVAL;
+  }
+  const int rc = check_arch("c6_forward_generic", board, layers, kernels, channels);
+  if (rc != C6_OK) return rc;
+  if (batch == 0) return C6_OK;
+  if (x == nullptr || conv_w == nullptr || pol_w == nullptr || workspace == nullptr ||
+      (value != nullptr && val_w == nullptr)) {
+    set_error("c6_forward_generic: null pointer (x, conv_w, pol_w, workspace, or value without val_w)");
+    return C6_EINVAL;
+  }
+  for (int l = 0; l < layers; ++l)
+    if (conv_w[l] == nullptr) {
+      set_error("c6_forward_generic: conv_w[%d] is null", l);
+      return C6_EINVAL;
+    }
+  if (workspace_bytes < generic_workspace_bytes(batch, board, layers, channels) ||
+      !aligned16(workspace)) {
+    set_error("c6_forward_generic: workspace too small or not 16-byte aligned");
+    return C6_EINVAL;
+  }
+  if (mask_mode < C6_MASK_NONE || mask_mode > C6_MASK_LEGAL ||
+      (mask_mode == C6_MASK_LEGAL && legal == nullptr)) {
+    set_error("c6_forward_generic: bad mask_mode %d", mask_mode);
+    return C6_EINVAL;
+  }
+  return launch_generic(x, x_dtype, batch, board, layers, kernels, channels, conv_w, conv_b,
+                        pol_w, pol_b, val_w, val_b, prec, workspace, logits, value, mask_mode,
+                        legal, fill, static_cast<hipStream_t>(stream));
 }
 
 int c6_mask_logits(const void *logits, const uint8_t *legal, int dtype, int64_t batch,

@@ -16,7 +16,7 @@ from typing import Any
 import torch
 
 from . import _lib
-from .model import _require_device_tensor, pack_state, run_forward
+from .model import _require_device_tensor, pack_state, run_forward, run_forward_generic
 
 
 @dataclass(slots=True)
@@ -107,35 +107,32 @@ class HistoricalPolicyEnsemble:
             return None
         return self._stack(states, key)
 
+    @property
+    def is_default_architecture(self) -> bool:
+        return (
+            self.board_size == 19
+            and self.kernels == (23, 3, 3, 3, 3, 3, 3, 3)
+            and self.channels == (32, 32, 64, 64, 64, 96, 96, 96)
+        )
+
+    def _model_state(self, m: int) -> dict[str, torch.Tensor]:
+        """Parameters of model ``m`` as the ensemble holds them (rounded to ``dtype``)."""
+        state = {}
+        for i in range(len(self.kernels)):
+            state[f"convs.{i}.weight"] = self.conv_weights[i][m]
+            if self.conv_biases[i] is not None:
+                state[f"convs.{i}.bias"] = self.conv_biases[i][m]
+        state["policy_output.weight"] = self.policy_weight[m]
+        if self.policy_bias is not None:
+            state["policy_output.bias"] = self.policy_bias[m]
+        return state
+
     def _packed_weights(self) -> torch.Tensor:
         if self._packed is None:
-            if self.device.type != "cuda":
-                raise RuntimeError(
-                    f"ensemble device is {self.device}: connect6_amd computes only on an MI355X "
-                    "(HIP) device; there is no CPU path"
-                )
-            default = (
-                self.board_size == 19
-                and self.kernels == (23, 3, 3, 3, 3, 3, 3, 3)
-                and self.channels == (32, 32, 64, 64, 64, 96, 96, 96)
-            )
-            if not default:
-                raise NotImplementedError(
-                    "the HIP kernels are built for the default architecture on a 19x19 board; got "
-                    f"board {self.board_size}, kernels {self.kernels}, channels {self.channels}"
-                )
             one = _lib.packed_bytes(self._prec)
             buf = torch.empty((self.num_models, one), dtype=torch.uint8, device=self.device)
             for m in range(self.num_models):
-                # the values packed are the ones the ensemble holds (already rounded to `dtype`)
-                state = {f"convs.{i}.weight": self.conv_weights[i][m] for i in range(8)}
-                for i in range(8):
-                    if self.conv_biases[i] is not None:
-                        state[f"convs.{i}.bias"] = self.conv_biases[i][m]
-                state["policy_output.weight"] = self.policy_weight[m]
-                if self.policy_bias is not None:
-                    state["policy_output.bias"] = self.policy_bias[m]
-                pack_state(state, self._prec, buf[m])
+                pack_state(self._model_state(m), self._prec, buf[m])
             self._packed = buf
         return self._packed
 
@@ -148,12 +145,25 @@ class HistoricalPolicyEnsemble:
                 f"bad history batch {tuple(x.shape)}; expected "
                 f"[{self.num_models}, T, {expected_tail[0]}, {expected_tail[1]}, {expected_tail[2]}]"
             )
-        packed = self._packed_weights()
+        if self.device.type != "cuda":
+            raise RuntimeError(
+                f"ensemble device is {self.device}: connect6_amd computes only on an MI355X "
+                "(HIP) device; there is no CPU path"
+            )
         if x.device != self.device or x.dtype != self.dtype:
             x = x.to(device=self.device, dtype=self.dtype, non_blocking=True)
         _require_device_tensor(x, "history input")
         m, t = int(x.shape[0]), int(x.shape[1])
-        logits, _, _, _ = run_forward(x.reshape(m * t, *expected_tail), packed, self._prec, m, t,
-                                      want_value=False)
+        if t == 0:
+            return torch.empty((m, 0, self.action_size), dtype=self.dtype, device=self.device)
+        if self.is_default_architecture:
+            logits, _, _, _ = run_forward(x.reshape(m * t, *expected_tail), self._packed_weights(),
+                                          self._prec, m, t, want_value=False)
+        else:  # other architectures: layer by layer, one model after the other
+            logits = torch.cat([
+                run_forward_generic(x[i], self._model_state(i), self.kernels, self.channels,
+                                    self._prec, want_value=False)[0]
+                for i in range(m)
+            ])
         logits = logits.view(m, t, self.action_size)
         return logits if self.dtype == torch.float32 else logits.to(self.dtype)

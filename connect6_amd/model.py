@@ -122,6 +122,71 @@ def run_forward(
     return logits, value, actions, logprob
 
 
+def run_forward_generic(
+    x: torch.Tensor,
+    state: dict[str, torch.Tensor],
+    kernels,
+    channels,
+    prec: int,
+    *,
+    want_value: bool = True,
+    mask_mode: int = _lib.MASK_NONE,
+    legal: torch.Tensor | None = None,
+    fill: float = _FILL_LOWEST,
+):
+    """Launch ``c6_forward_generic`` for one weight set of any architecture:
+    x ``[B,3,n,n]`` -> (logits ``[B,n*n]``, value ``[B]`` or None)."""
+    lib = _lib.load()
+    dev = x.device
+    x = x.contiguous()
+    b, n = int(x.shape[0]), int(x.shape[-1])
+    layers = len(kernels)
+    keep = []
+
+    def dev32(key, required=True):
+        if key not in state:
+            if required:
+                raise KeyError(f"missing parameter {key}")
+            return None
+        t = state[key].detach().to(device=dev, dtype=torch.float32).contiguous()
+        keep.append(t)
+        return t
+
+    ws = [dev32(f"convs.{i}.weight") for i in range(layers)]
+    bs = [dev32(f"convs.{i}.bias", required=False) for i in range(layers)]
+    pw, pb = dev32("policy_output.weight"), dev32("policy_output.bias", required=False)
+    vw = dev32("value_output.weight", required=False) if want_value else None
+    vb = dev32("value_output.bias", required=False) if want_value else None
+    ints = ctypes.c_int * layers
+    ck, cc = ints(*[int(k) for k in kernels]), ints(*[int(c) for c in channels])
+    vp = ctypes.c_void_p
+    wptrs = (vp * layers)(*[t.data_ptr() for t in ws])
+    bptrs = (vp * layers)(*[(t.data_ptr() if t is not None else None) for t in bs])
+    nbytes = ctypes.c_size_t(0)
+    _lib.check(lib.c6_generic_workspace_bytes(b, n, layers, cc, ctypes.byref(nbytes)),
+               "c6_generic_workspace_bytes")
+    workspace = torch.empty(max(int(nbytes.value), 16), dtype=torch.uint8, device=dev)
+    logits = torch.empty((b, n * n), dtype=torch.float32, device=dev)
+    value = torch.empty((b,), dtype=torch.float32, device=dev) if want_value else None
+    if legal is not None:
+        if legal.shape != (b, n * n):
+            raise ValueError(f"legal mask must have shape ({b}, {n * n}), got {tuple(legal.shape)}")
+        legal = legal.to(dev).contiguous()
+        legal = legal.view(torch.uint8) if legal.dtype == torch.bool else legal
+
+    def ptr(t):
+        return t.data_ptr() if t is not None else None
+
+    with torch.cuda.device(dev):
+        rc = lib.c6_forward_generic(x.data_ptr(), _lib.torch_dtype_code(x.dtype), b, n, layers, ck,
+                                    cc, wptrs, bptrs, ptr(pw), ptr(pb), ptr(vw), ptr(vb), prec,
+                                    workspace.data_ptr(), workspace.numel(), ptr(logits),
+                                    ptr(value), mask_mode, ptr(legal), fill,
+                                    _lib.stream_ptr(dev))
+    _lib.check(rc, "c6_forward_generic")
+    return logits, value
+
+
 class PolicyValueNet(nn.Module):
     """Fully convolutional policy + value network for Connect6
     (reference: connect6/model.py:9-111).
@@ -265,16 +330,19 @@ class PolicyValueNet(nn.Module):
                 "torch.no_grad() / torch.inference_mode() (training stays on a PyTorch module "
                 "sharing this state_dict)"
             )
-        if not self.is_default_architecture:
-            raise NotImplementedError(
-                "the HIP kernels are built for board 19, kernels "
-                f"{self.DEFAULT_KERNELS}, channels {self.DEFAULT_CHANNELS}; got board "
-                f"{self.board_size}, kernels {self.kernels}, channels {self.channels}"
-            )
+
+    def _generic(self, x, prec, **kw):
+        """Non-default architectures run layer by layer (``c6_forward_generic``)."""
+        if int(x.shape[0]) == 0:
+            return (torch.empty((0, self.action_size), dtype=torch.float32, device=x.device),
+                    torch.empty((0,), dtype=torch.float32, device=x.device))
+        return run_forward_generic(x, self.state_dict(), self.kernels, self.channels, prec, **kw)
 
     def forward(self, x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
         self._check_input(x)
         prec = self.resolve_precision()
+        if not self.is_default_architecture:
+            return self._generic(x, prec)
         logits, value, _, _ = run_forward(x, self.packed_weights(prec), prec, 1, int(x.shape[0]))
         return logits, value
 
@@ -290,10 +358,13 @@ class PolicyValueNet(nn.Module):
         non-zero there.  ``fill`` defaults to ``finfo(float32).min``."""
         self._check_input(x)
         prec = self.resolve_precision()
+        mask_mode = _lib.MASK_INPUT if legal is None else _lib.MASK_LEGAL
+        fill = _FILL_LOWEST if fill is None else float(fill)
+        if not self.is_default_architecture:
+            return self._generic(x, prec, mask_mode=mask_mode, legal=legal, fill=fill)
         logits, value, _, _ = run_forward(
             x, self.packed_weights(prec), prec, 1, int(x.shape[0]),
-            mask_mode=_lib.MASK_INPUT if legal is None else _lib.MASK_LEGAL, legal=legal,
-            fill=_FILL_LOWEST if fill is None else float(fill),
+            mask_mode=mask_mode, legal=legal, fill=fill,
         )
         return logits, value
 
@@ -311,6 +382,11 @@ class PolicyValueNet(nn.Module):
         reference (connect6/train.py:195-203) without materialising logits.
         Returns ``(actions int64[B], logprob[B], value[B])`` (+ masked logits)."""
         self._check_input(x)
+        if not self.is_default_architecture:
+            raise NotImplementedError(
+                "the fused self-play step is built for the default architecture on a 19x19 board; "
+                "use forward_masked() followed by sample_actions() elsewhere"
+            )
         prec = self.resolve_precision()
         logits, value, actions, logprob = run_forward(
             x, self.packed_weights(prec), prec, 1, int(x.shape[0]), want_logits=return_logits,

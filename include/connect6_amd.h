@@ -87,6 +87,25 @@ int c6_forward(const void *x, int x_dtype, int64_t groups, int64_t boards_per_gr
                const float *u, float temperature, int64_t *actions, float *logprob,
                void *stream);
 
+/* Forward of ONE weight set for any architecture the reference's PolicyValueNet accepts
+ * (connect6/model.py:26-77: any board size, odd kernels, positive channel counts), layer by
+ * layer through a caller-provided workspace.  Compatibility path for non-default
+ * architectures (the reference's own tests use board 5, kernels 3,3,3, channels 8,8,16);
+ * the default architecture should use c6_forward.
+ *   x        device [B,3,n,n] of element type x_dtype
+ *   kernels, channels: HOST arrays of `layers` ints
+ *   conv_w / conv_b:   HOST arrays of `layers` device fp32 pointers (PyTorch layouts)
+ *   workspace: device, c6_generic_workspace_bytes(...) bytes, 16-byte aligned
+ *   logits fp32 [B,n*n] (may be NULL), value fp32 [B] (may be NULL; val_w may then be NULL) */
+int c6_generic_workspace_bytes(int64_t batch, int board, int layers, const int *channels,
+                               size_t *bytes);
+int c6_forward_generic(const void *x, int x_dtype, int64_t batch, int board, int layers,
+                       const int *kernels, const int *channels, const float *const *conv_w,
+                       const float *const *conv_b, const float *pol_w, const float *pol_b,
+                       const float *val_w, const float *val_b, int prec, void *workspace,
+                       size_t workspace_bytes, float *logits, float *value, int mask_mode,
+                       const uint8_t *legal, float fill, void *stream);
+
 /* Out-of-place occupied-square masking of existing logits.
  * Replaces: mask_logits (connect6/model.py:123-125).
  * logits/out: device [B,361] of element type dtype; legal: device uint8 [B,361];

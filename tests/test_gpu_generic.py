@@ -1,0 +1,84 @@
+"""Non-default architectures (any board / kernels / channels the reference's
+PolicyValueNet accepts) run through the layer-by-layer HIP path."""
+from pathlib import Path
+
+import pytest
+import torch
+
+import connect6_amd as c6
+from oracle import cref
+from oracle import torch_ref as R
+from tests.util import rel_l2
+
+pytestmark = pytest.mark.gpu
+
+
+def test_grouped_history_matches_individual_models_reference_test_shape(cuda):
+    # tests/test_training_features.py:120-151 of the reference, on the GPU
+    torch.manual_seed(123)
+    board_size = 5
+    model_cfg = {"architecture_version": 4, "kernels": [3, 3, 3], "channels": [8, 8, 16],
+                 "compile": False, "compile_mode": "default"}
+    game_cfg = {"board_size": board_size, "win_length": 3}
+    models = [c6.build_model(model_cfg, board_size).to(cuda) for _ in range(2)]
+    checkpoints = [
+        c6.HistoricalCheckpoint(path=Path(f"model_update_{i + 1:08d}.pt"), update=i + 1,
+                                model_state=model.state_dict(), model_config=model_cfg,
+                                game_config=game_cfg)
+        for i, model in enumerate(models)
+    ]
+    ensemble = c6.HistoricalPolicyEnsemble(checkpoints, cuda)
+    x = torch.randn(2, 5, 3, board_size, board_size)
+    with torch.inference_mode():
+        grouped = ensemble.forward_grouped(x.to(cuda))
+        assert grouped.shape == (2, 5, 25)
+        for i, model in enumerate(models):
+            model.eval()
+            got, value = model(x[i].to(cuda))
+            assert torch.allclose(grouped[i], got, atol=1e-5, rtol=1e-5)
+            state = {k: v.cpu() for k, v in model.state_dict().items()}
+            expected, vexp = R.forward(state, x[i])
+            assert torch.allclose(grouped[i].cpu(), expected, atol=1e-5, rtol=1e-5)
+            assert torch.allclose(value.cpu(), vexp, atol=1e-5, rtol=1e-5)
+            assert torch.all(value <= 1) and torch.all(value >= -1)
+
+
+@pytest.mark.parametrize("board,kernels,channels", [(9, [5, 3, 1], [16, 24, 7]), (19, [7, 3], [5, 33])])
+def test_other_architectures_match_oracle_and_bruteforce(cuda, board, kernels, channels):
+    st = R.init_state(11, "torch_default", kernels=kernels, channels=channels)
+    model = c6.PolicyValueNet(board_size=board, kernels=kernels, channels=channels).to(cuda).eval()
+    model.load_state_dict(st)
+    assert not model.is_default_architecture
+    x = torch.randn(6, 3, board, board, generator=torch.Generator().manual_seed(3))
+    x[:, :2] = (x[:, :2] > 0.8).float()                    # stone planes
+    legal = ((x[:, 0] == 0) & (x[:, 1] == 0)).flatten(1)
+    with torch.inference_mode():
+        lo, vo = R.forward(st, x)
+        lc, vc = cref.forward(st, x[:2])
+        lg, vg = model(x.to(cuda))
+        lm, _ = model.forward_masked(x.to(cuda))
+        ll, _ = model.forward_masked(x.to(cuda), legal.to(cuda), fill=float("-inf"))
+    assert lg.shape == (6, board * board) and vg.shape == (6,)
+    assert rel_l2(lg, lo) <= 1e-5 and rel_l2(vg, vo) <= 1e-5
+    assert rel_l2(lg[:2], lc) <= 1e-5 and rel_l2(vg[:2], vc) <= 1e-5
+    assert torch.equal(lm.cpu(), R.mask_logits(lg.cpu(), legal))            # bit-exact fill / pass-through
+    assert torch.equal(torch.isneginf(ll.cpu()), ~legal)
+    # 16-bit contracts: same roundings as the emulation in the oracle
+    model.precision = "bf16"
+    with torch.inference_mode():
+        lb, vb = model(x.to(cuda))
+        le, ve = R.forward_bf16_emulated(st, x)
+    assert rel_l2(lb, le) <= 2e-3 and rel_l2(lb, lo) <= 2e-2 and rel_l2(vb, vo) <= 2e-2
+
+
+def test_generic_path_edge_cases(cuda):
+    model = c6.PolicyValueNet(board_size=5, kernels=[3], channels=[4]).to(cuda).eval()
+    with torch.inference_mode():
+        logits, value = model(torch.zeros(0, 3, 5, 5, device=cuda))
+        assert logits.shape == (0, 25) and value.shape == (0,)
+        logits, value = model(torch.zeros(3, 3, 5, 5, device=cuda))     # tests/test_model.py:11-18
+        assert torch.count_nonzero(logits) == 0 and torch.count_nonzero(value) == 0
+        with pytest.raises(NotImplementedError):
+            model.selfplay_step(torch.zeros(1, 3, 5, 5, device=cuda), torch.zeros(1, device=cuda))
+    with pytest.raises(ValueError):
+        model(torch.zeros(2, 3, 6, 6, device=cuda))

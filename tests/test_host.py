@@ -56,6 +56,19 @@ def test_entry_points_reject_bad_arguments_before_touching_the_device():
     assert lib.c6_d4_expand(None, 0, 2, None, None) == -1
     assert lib.c6_d4_reduce(None, None, 2, None, None, None) == -1
     assert lib.c6_pack_weights(None, None, None, None, None, None, 1, None, None) == -1
+    n = ctypes.c_size_t(0)
+    ch = (ctypes.c_int * 3)(8, 8, 16)
+    ks = (ctypes.c_int * 3)(3, 3, 3)
+    assert lib.c6_generic_workspace_bytes(4, 5, 3, ch, ctypes.byref(n)) == 0
+    assert n.value == 2 * 4 * 16 * 25 * 4
+    assert lib.c6_generic_workspace_bytes(4, 0, 3, ch, ctypes.byref(n)) == -1
+    bad = (ctypes.c_int * 3)(3, 4, 3)      # even kernel, as connect6/model.py:44-45 rejects
+    assert lib.c6_forward_generic(None, 0, 2, 5, 3, bad, ch, None, None, None, None, None, None, 0,
+                                  None, 0, None, None, 0, None, 0.0, None) == -1
+    assert lib.c6_forward_generic(None, 0, 2, 5, 3, ks, ch, None, None, None, None, None, None, 0,
+                                  None, 0, None, None, 0, None, 0.0, None) == -1
+    assert lib.c6_forward_generic(None, 0, 0, 5, 3, ks, ch, None, None, None, None, None, None, 0,
+                                  None, 0, None, None, 0, None, 0.0, None) == 0
 
 
 def test_model_attributes_match_reference_contract():
