@@ -181,25 +181,40 @@ def main() -> int:
         td = timed(lambda: c6.evaluate_d4(model, xd), steps=5, warmup=2)
         out["d4_eval_8192x8"] = {"base_boards_per_s": 8192 / td, "ms": td * 1e3}
 
-        # ---- HBM-bound tail kernels: algorithmic bytes / time ----
-        nb = 65536
+        # ---- HBM-bound tail kernels: algorithmic bytes / kernel time (HIP events) ----
+        def event_timed(fn, steps=20, warmup=3):
+            with torch.inference_mode():
+                for _ in range(warmup):
+                    fn()
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(steps):
+                    fn()
+                e1.record()
+                torch.cuda.synchronize()
+            return e0.elapsed_time(e1) * 1e-3 / steps
+
+        nb, nd = 262144, 32768          # large enough that launch overhead does not show
         lg = torch.randn(nb, 361, device=dev)
         lgl = gen_boards(nb, 300, 5)[1].to(dev)
         un = gen_uniform(nb, 3).to(dev)
-        views = torch.randn(8, 8192, 361, device=dev)
-        vals = torch.randn(8, 8192, device=dev)
+        xdd = gen_boards(nd, 200, 9)[0].to(dev)
+        views = torch.randn(8, nd, 361, device=dev)
+        vals = torch.randn(8, nd, device=dev)
         hbm = {}
-        t = timed(lambda: c6.mask_logits(lg, lgl), steps=20)
-        hbm["mask_logits_f32"] = {"GBps": nb * 361 * (4 + 1 + 4) / t / 1e9}
-        t = timed(lambda: c6.sample_actions(lg, lgl, 1.0, un), steps=20)
-        hbm["softmax_sample"] = {"GBps": nb * (361 * 5 + 4 + 12) / t / 1e9}
-        t = timed(lambda: c6.d4_expand(xd), steps=20)
-        hbm["d4_expand_f32"] = {"GBps": 8192 * 3 * 361 * 4 * 9 / t / 1e9}
-        t = timed(lambda: c6.d4_reduce(views, vals), steps=20)
-        hbm["d4_reduce"] = {"GBps": 8192 * (361 * 4 * 9 + 4 * 9) / t / 1e9}
+        t = event_timed(lambda: c6.mask_logits(lg, lgl))
+        hbm["mask_logits_f32"] = {"GBps": nb * 361 * (4 + 1 + 4) / t / 1e9, "boards": nb}
+        t = event_timed(lambda: c6.sample_actions(lg, lgl, 1.0, un))
+        hbm["softmax_sample"] = {"GBps": nb * (361 * 5 + 4 + 12) / t / 1e9, "boards": nb}
+        t = event_timed(lambda: c6.d4_expand(xdd))
+        hbm["d4_expand_f32"] = {"GBps": nd * 3 * 361 * 4 * 9 / t / 1e9, "boards": nd}
+        t = event_timed(lambda: c6.d4_reduce(views, vals))
+        hbm["d4_reduce"] = {"GBps": nd * (361 * 4 * 9 + 4 * 9) / t / 1e9, "boards": nd}
         for v in hbm.values():
             v["frac_of_hbm_peak"] = v["GBps"] / HBM_PEAK_GBS
         out["hbm_kernels"] = hbm
+        del lg, lgl, un, xdd, views, vals
 
     if not args.no_cpu_baseline:
         # The PyTorch fp32 oracle (the checker) on this box's host cores, configs[0] shape.

@@ -52,64 +52,180 @@ __global__ void mask2_kernel(const uint16_t *__restrict__ in, const uint8_t *__r
   }
 }
 
-// One wave per board: masked softmax over 361 logits and inverse-CDF draw
-// (connect6/train.py:195-213 of the reference, with the uniform supplied).
+// Rows of 361 elements are only 4-byte aligned, but FOUR consecutive rows span 4*361*4 =
+// 16*361 bytes and start 16-byte aligned (the tensor base is).  The kernels below therefore
+// work on groups of four boards (eight planes for the view gather) and move them with 16-byte
+// accesses; the last, partial group falls back to element accesses.
+__device__ __forceinline__ void copy_span_f32(float *dst_lds, const float *__restrict__ src,
+                                              int n_full4, int n_elems, bool vec) {
+  if (vec) {
+    for (int i = threadIdx.x; i < n_full4; i += blockDim.x)
+      reinterpret_cast<f32x4 *>(dst_lds)[i] = reinterpret_cast<const f32x4 *>(src)[i];
+  } else {
+    for (int i = threadIdx.x; i < n_elems; i += blockDim.x) dst_lds[i] = src[i];
+  }
+}
+
+// Eight boards per workgroup (two per wave): masked softmax over 361 logits and inverse-CDF
+// draw (connect6/train.py:195-213 of the reference, with the uniform supplied).  All eight
+// rows are requested up front so that enough bytes are in flight per CU to cover HBM latency.
+constexpr int kSampleBoards = 8;
 __global__ __launch_bounds__(256) void sample_kernel(const float *__restrict__ logits,
                                                      const uint8_t *__restrict__ legal,
                                                      const float *__restrict__ u,
                                                      float inv_temperature, long long batch,
                                                      long long *__restrict__ actions,
                                                      float *__restrict__ logprob) {
-  const int lane = threadIdx.x & 63;
-  const long long b = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (b >= batch) return;
-  const float *row = logits + (size_t)b * kPix;
-  const uint8_t *lrow = legal ? legal + (size_t)b * kPix : nullptr;
-  int a;
-  float lp;
-  wave_sample(
-      lane, u[b], [&](int i) { return row[i] * inv_temperature; },
-      [&](int i) { return lrow ? lrow[i] != 0 : true; }, a, lp);
-  if (lane == 0) {
-    actions[b] = a;
-    if (logprob) logprob[b] = lp;
+  __shared__ __attribute__((aligned(16))) float s_logit[kSampleBoards * kPix];
+  __shared__ __attribute__((aligned(16))) uint8_t s_legal[kSampleBoards * kPix];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const long long b0 = (long long)blockIdx.x * kSampleBoards;
+  const int nb = (int)(batch - b0 < kSampleBoards ? batch - b0 : kSampleBoards);
+  const bool full = nb == kSampleBoards;
+  copy_span_f32(s_logit, logits + (size_t)b0 * kPix, kSampleBoards * kPix / 4, nb * kPix,
+                full && (reinterpret_cast<uintptr_t>(logits) & 15u) == 0);
+  if (legal != nullptr) {
+    const uint8_t *lsrc = legal + (size_t)b0 * kPix;  // 8*361 bytes: an 8-byte aligned span
+    if (full && (reinterpret_cast<uintptr_t>(legal) & 7u) == 0) {
+      for (int i = threadIdx.x; i < kSampleBoards * kPix / 8; i += blockDim.x)
+        reinterpret_cast<v2i *>(s_legal)[i] = reinterpret_cast<const v2i *>(lsrc)[i];
+    } else {
+      for (int i = threadIdx.x; i < nb * kPix; i += blockDim.x) s_legal[i] = lsrc[i];
+    }
+  }
+  __syncthreads();
+  const bool masked = legal != nullptr;
+#pragma unroll
+  for (int r = 0; r < kSampleBoards / 4; ++r) {
+    const int bl = w + 4 * r;
+    if (bl < nb) {
+      const float *row = s_logit + bl * kPix;
+      const uint8_t *lrow = s_legal + bl * kPix;
+      int a;
+      float lp;
+      wave_sample(
+          lane, u[b0 + bl], [&](int i) { return row[i] * inv_temperature; },
+          [&](int i) { return masked ? lrow[i] != 0 : true; }, a, lp);
+      if (lane == 0) {
+        actions[b0 + bl] = a;
+        if (logprob) logprob[b0 + bl] = lp;
+      }
+    }
   }
 }
 
-// out[p,b,ch,v] = x[b,ch,from_view(v,p)]   (connect6/train.py:222-230)
+// out[p,plane,v] = x[plane, from_view(v,p)]   (connect6/train.py:222-230)
+// grid.y = view; each workgroup stages eight planes in LDS and writes the permuted planes.
+constexpr int kExpandPlanes = 8;
 template <typename T>
-__global__ void d4_expand_kernel(const T *__restrict__ x, long long batch, T *__restrict__ out) {
-  const long long per_view = batch * 3 * kPix;
-  const long long n = 8 * per_view;
-  const long long stride = (long long)gridDim.x * blockDim.x;
-  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
-    const int p = (int)(i / per_view);
-    const long long rem = i - (long long)p * per_view;
-    const long long plane = rem / kPix;
-    const int v = (int)(rem - plane * kPix);
-    out[i] = x[plane * kPix + d4_from_view(v, p)];
+__global__ __launch_bounds__(256) void d4_expand_kernel(const T *__restrict__ x, long long planes,
+                                                        T *__restrict__ out) {
+  constexpr int VEC = 16 / sizeof(T);                       // elements per 16-byte access
+  constexpr int SPAN = kExpandPlanes * kPix;                // 2888 elements: a multiple of VEC
+  static_assert(SPAN % VEC == 0, "eight planes must be whole 16-byte units");
+  typedef T vec_t __attribute__((ext_vector_type(VEC)));
+  __shared__ __attribute__((aligned(16))) T s_in[SPAN];
+  __shared__ unsigned short s_map[kPix];
+  const int p = blockIdx.y;
+  const long long plane0 = (long long)blockIdx.x * kExpandPlanes;
+  const int np = (int)((planes - plane0) < kExpandPlanes ? (planes - plane0) : kExpandPlanes);
+  for (int v = threadIdx.x; v < kPix; v += blockDim.x) s_map[v] = (unsigned short)d4_from_view(v, p);
+  const T *src = x + plane0 * kPix;
+  T *dst = out + ((size_t)p * planes + plane0) * kPix;
+  const bool aligned = ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u) == 0;
+  if (np == kExpandPlanes && aligned) {
+    for (int i = threadIdx.x; i < SPAN / VEC; i += blockDim.x)
+      reinterpret_cast<vec_t *>(s_in)[i] = reinterpret_cast<const vec_t *>(src)[i];
+    __syncthreads();
+    for (int i = threadIdx.x; i < SPAN / VEC; i += blockDim.x) {
+      vec_t o;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        const int idx = i * VEC + e;
+        const int pl = idx / kPix, v = idx - pl * kPix;
+        o[e] = s_in[pl * kPix + s_map[v]];
+      }
+      reinterpret_cast<vec_t *>(dst)[i] = o;
+    }
+  } else {
+    for (int i = threadIdx.x; i < np * kPix; i += blockDim.x) s_in[i] = src[i];
+    __syncthreads();
+    for (int i = threadIdx.x; i < np * kPix; i += blockDim.x) {
+      const int pl = i / kPix, v = i - pl * kPix;
+      dst[i] = s_in[pl * kPix + s_map[v]];
+    }
   }
 }
 
 // logits[b,a] = mean_p view_logits[p,b,to_view(a,p)]; values[b] = mean_p view_values[p,b]
-__global__ void d4_reduce_kernel(const float *__restrict__ vl, const float *__restrict__ vv,
-                                 long long batch, float *__restrict__ logits,
-                                 float *__restrict__ values) {
-  const long long n = batch * kPix;
-  const long long stride = (long long)gridDim.x * blockDim.x;
-  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
-    const long long b = i / kPix;
-    const int a = (int)(i - b * kPix);
+// Four boards per workgroup; the eight views stream through a double buffer in LDS (the next
+// view's rows are in flight while the current one is gathered), accumulators stay in registers.
+__global__ __launch_bounds__(256) void d4_reduce_kernel(const float *__restrict__ vl,
+                                                        const float *__restrict__ vv,
+                                                        long long batch,
+                                                        float *__restrict__ logits,
+                                                        float *__restrict__ values) {
+  constexpr int SPAN = 4 * kPix;            // 1444 floats = 361 16-byte units
+  constexpr int PER = (SPAN + 255) / 256;   // outputs per thread
+  __shared__ __attribute__((aligned(16))) float s_v[2][SPAN];
+  const long long b0 = (long long)blockIdx.x * 4;
+  const int nb = (int)(batch - b0 < 4 ? batch - b0 : 4);
+  const int n = nb * kPix;
+  const bool vec = nb == 4 && (batch & 3) == 0 && (reinterpret_cast<uintptr_t>(vl) & 15u) == 0;
+  const int t = threadIdx.x;
+  f32x4 stage[2];
+  float stage1[PER];
+  auto fetch = [&](int p) {
+    const float *src = vl + ((size_t)p * batch + b0) * kPix;
+    if (vec) {
+      stage[0] = reinterpret_cast<const f32x4 *>(src)[t];
+      if (t + 256 < kPix) stage[1] = reinterpret_cast<const f32x4 *>(src)[t + 256];
+    } else {
+#pragma unroll
+      for (int k = 0; k < PER; ++k)
+        if (t + 256 * k < n) stage1[k] = src[t + 256 * k];
+    }
+  };
+  auto commit = [&](int buf) {
+    if (vec) {
+      reinterpret_cast<f32x4 *>(s_v[buf])[t] = stage[0];
+      if (t + 256 < kPix) reinterpret_cast<f32x4 *>(s_v[buf])[t + 256] = stage[1];
+    } else {
+#pragma unroll
+      for (int k = 0; k < PER; ++k)
+        if (t + 256 * k < n) s_v[buf][t + 256 * k] = stage1[k];
+    }
+  };
+  int bl[PER], a[PER];
+  float acc[PER];
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    const int i = t + 256 * k;
+    bl[k] = i / kPix;
+    a[k] = i - bl[k] * kPix;
+    acc[k] = 0.0f;
+  }
+  fetch(0);
+  commit(0);
+  __syncthreads();
+#pragma unroll
+  for (int p = 0; p < 8; ++p) {
+    if (p < 7) fetch(p + 1);
+#pragma unroll
+    for (int k = 0; k < PER; ++k)
+      if (t + 256 * k < n) acc[k] += s_v[p & 1][bl[k] * kPix + d4_to_view(a[k], p)];
+    if (p < 7) commit((p + 1) & 1);
+    __syncthreads();
+  }
+  float *dst = logits + (size_t)b0 * kPix;
+#pragma unroll
+  for (int k = 0; k < PER; ++k)
+    if (t + 256 * k < n) dst[t + 256 * k] = acc[k] * 0.125f;
+  if (t < nb && values != nullptr) {
     float s = 0.0f;
 #pragma unroll
-    for (int p = 0; p < 8; ++p) s += vl[((size_t)p * batch + b) * kPix + d4_to_view(a, p)];
-    logits[i] = s * 0.125f;
-    if (a == 0 && values != nullptr) {
-      float t = 0.0f;
-#pragma unroll
-      for (int p = 0; p < 8; ++p) t += vv[(size_t)p * batch + b];
-      values[b] = t * 0.125f;
-    }
+    for (int p = 0; p < 8; ++p) s += vv[(size_t)p * batch + b0 + t];
+    values[b0 + t] = s * 0.125f;
   }
 }
 
@@ -144,25 +260,26 @@ int launch_mask(const void *logits, const uint8_t *legal, int elem_bytes, long l
 
 int launch_sample(const float *logits, const uint8_t *legal, const float *u, float inv_t,
                   long long batch, long long *actions, float *logprob, hipStream_t st) {
-  hipLaunchKernelGGL(sample_kernel, dim3((unsigned)((batch + 3) / 4)), dim3(256), 0, st, logits,
+  hipLaunchKernelGGL(sample_kernel, dim3((unsigned)((batch + kSampleBoards - 1) / kSampleBoards)), dim3(256), 0, st, logits,
                      legal, u, inv_t, batch, actions, logprob);
   return check_launch("softmax_sample");
 }
 
 int launch_d4_expand(const void *x, int elem_bytes, long long batch, void *out, hipStream_t st) {
-  const long long n = 8 * batch * 3 * kPix;
+  const long long planes = batch * 3;
+  const dim3 grid((unsigned)((planes + kExpandPlanes - 1) / kExpandPlanes), 8);
   if (elem_bytes == 4)
-    hipLaunchKernelGGL(d4_expand_kernel<uint32_t>, dim3(grid_for(n, 256)), dim3(256), 0, st,
-                       (const uint32_t *)x, batch, (uint32_t *)out);
+    hipLaunchKernelGGL(d4_expand_kernel<uint32_t>, grid, dim3(256), 0, st, (const uint32_t *)x,
+                       planes, (uint32_t *)out);
   else
-    hipLaunchKernelGGL(d4_expand_kernel<uint16_t>, dim3(grid_for(n, 256)), dim3(256), 0, st,
-                       (const uint16_t *)x, batch, (uint16_t *)out);
+    hipLaunchKernelGGL(d4_expand_kernel<uint16_t>, grid, dim3(256), 0, st, (const uint16_t *)x,
+                       planes, (uint16_t *)out);
   return check_launch("d4_expand");
 }
 
 int launch_d4_reduce(const float *vl, const float *vv, long long batch, float *logits,
                      float *values, hipStream_t st) {
-  hipLaunchKernelGGL(d4_reduce_kernel, dim3(grid_for(batch * kPix, 256)), dim3(256), 0, st, vl, vv,
+  hipLaunchKernelGGL(d4_reduce_kernel, dim3((unsigned)((batch + 3) / 4)), dim3(256), 0, st, vl, vv,
                      batch, logits, values);
   return check_launch("d4_reduce");
 }
