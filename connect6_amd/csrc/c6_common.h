@@ -59,29 +59,48 @@ struct PrecF32 {
   static constexpr int ID = C6_PREC_F32;
   static constexpr int EB = 4;        // bytes per element
   static constexpr int SPLIT = 0;
+  static constexpr int LO8 = 0;
 };
 struct PrecBF16 {
   static constexpr int ID = C6_PREC_BF16;
   static constexpr int EB = 2;
   static constexpr int SPLIT = 0;
+  static constexpr int LO8 = 0;
 };
 struct PrecF16 {
   static constexpr int ID = C6_PREC_F16;
   static constexpr int EB = 2;
   static constexpr int SPLIT = 0;
+  static constexpr int LO8 = 0;
 };
 struct PrecBF16X2 {
   static constexpr int ID = C6_PREC_BF16X2;
   static constexpr int EB = 2;
-  static constexpr int SPLIT = 1;     // activations stored as hi plane + lo plane
+  static constexpr int SPLIT = 1;     // activations stored as hi plane + lo plane, both bf16
+  static constexpr int LO8 = 0;
 };
+struct PrecBF16F8 {
+  static constexpr int ID = C6_PREC_BF16F8;
+  static constexpr int EB = 2;
+  static constexpr int SPLIT = 0;
+  static constexpr int LO8 = 1;       // bf16 plane + the dropped low-order part as scaled fp8
+};
+
+// bf16 + fp8 mode: what rounding an activation to bf16 drops (|lo| <= 2^-9 |a|) is kept as
+// e4m3 scaled by 2^kLoScaleLog2 and contracted with an e4m3 copy of the weights in a second
+// pass of v_mfma_scale_f32_32x32x64_f8f6f4 (K = 64 per instruction at twice the bf16 rate).
+// The weight copy of layer l is scaled by 2^sw[l] (sw in the packed tail, from max|w|); the
+// instruction's block scales undo both factors.
+constexpr int kLoScaleLog2 = 12;
+constexpr int kLoRing = 3;            // fp8 weight prefetch depth (64-wide K chunks)
 
 template <class P> struct Geo {
   static constexpr int EB = P::EB;
   static constexpr int E = 16 / EB;                 // elements per 16-byte fragment lane
   static constexpr int KSTEP = 2 * E;               // K elements contracted per fragment pair
   static constexpr int PLANE = kChSlots * EB;       // bytes of one precision plane of a position
-  static constexpr int RECB = PLANE * (P::SPLIT ? 2 : 1);  // payload bytes per position
+  static constexpr int LO_OFF = PLANE;              // fp8 low-order bytes follow the bf16 plane
+  static constexpr int RECB = PLANE * (P::SPLIT ? 2 : 1) + (P::LO8 ? kChSlots : 0);  // payload bytes
   // LDS bank conflicts: a ds_read_b128 is served 16 lanes at a time, so 16 consecutive
   // positions must land on 16 different 16-byte bank groups.  192-byte records get there
   // with 16 bytes of padding (stride 208 = 13 x 16); 384-byte records (fp32, hi+lo) would
@@ -107,10 +126,24 @@ template <class P> struct Geo {
     for (int i = 0; i < l; ++i) s += layer_frags(i);
     return s;
   }
-  static constexpr int TOTAL_FRAGS = frag_offset(8) + kOverreadFrags;
+  static constexpr int HI_FRAGS = frag_offset(8) + kOverreadFrags;
+  // fp8 copy of the 3x3 layers' weights (LO8 mode only).  K is cut into half-chunks of 32
+  // channels of one tap; a 64-wide chunk is two consecutive half-chunks, one per lane half.
+  // Fragment (chunk, cout tile, piece) = 64 lanes x 16 B; a lane's 32 bytes are pieces 0 and 1.
+  static constexpr int lo_half_chunks(int l) { return 9 * kCinArr[l] / 32; }
+  static constexpr int lo_chunks(int l) { return (lo_half_chunks(l) + 1) / 2; }
+  static constexpr int lo_layer_frags(int l) { return l == 0 ? 0 : lo_chunks(l) * (kCoutArr[l] / 32) * 2; }
+  static constexpr int lo_frag_offset(int l) {  // in 1 KiB fragments, from the start of the buffer
+    int s = HI_FRAGS;
+    for (int i = 0; i < l; ++i) s += lo_layer_frags(i);
+    return s;
+  }
+  static constexpr int LO_FRAGS = P::LO8 ? (lo_frag_offset(8) - HI_FRAGS) + kLoRing * 3 * 2 : 0;
+  static constexpr int TOTAL_FRAGS = HI_FRAGS + LO_FRAGS;
   static constexpr size_t TAIL_OFF = (size_t)TOTAL_FRAGS * 1024;  // fp32 tail: biases, heads
-  // tail floats: bias[544] polw[96] valw[96] polb valb (+pad)
-  static constexpr int TAIL_FLOATS = kBiasTotal + 2 * kHeadC + 4;
+  // tail words: bias[544] polw[96] valw[96] polb valb pad pad, then 8 ints sw[layer]
+  static constexpr int TAIL_SW = kBiasTotal + 2 * kHeadC + 4;
+  static constexpr int TAIL_FLOATS = TAIL_SW + 8;
   static constexpr size_t PACKED_BYTES = TAIL_OFF + (size_t)TAIL_FLOATS * 4;
 };
 

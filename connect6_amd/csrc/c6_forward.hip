@@ -41,6 +41,9 @@ template <> __device__ __forceinline__ void mma<PrecBF16>(const v4i &a, const v4
 template <> __device__ __forceinline__ void mma<PrecBF16X2>(const v4i &a, const v4i &b, f32x16 &c) {
   mma<PrecBF16>(a, b, c);
 }
+template <> __device__ __forceinline__ void mma<PrecBF16F8>(const v4i &a, const v4i &b, f32x16 &c) {
+  mma<PrecBF16>(a, b, c);
+}
 template <> __device__ __forceinline__ void mma<PrecF16>(const v4i &a, const v4i &b, f32x16 &c) {
   c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
                                              __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
@@ -105,6 +108,15 @@ template <class P> __device__ __forceinline__ Packed4<P> pack4(const float (&v)[
       r.lo[0] = pack2<P>(v[0] - bf16_lo(r.hi[0]), v[1] - bf16_hi(r.hi[0]));
       r.lo[1] = pack2<P>(v[2] - bf16_lo(r.hi[1]), v[3] - bf16_hi(r.hi[1]));
     }
+    if constexpr (P::LO8) {  // dropped low-order parts, scaled, as four e4m3 bytes
+      constexpr float S = (float)(1 << kLoScaleLog2);
+      const float l0 = __builtin_amdgcn_fmed3f((v[0] - bf16_lo(r.hi[0])) * S, -448.0f, 448.0f);
+      const float l1 = __builtin_amdgcn_fmed3f((v[1] - bf16_hi(r.hi[0])) * S, -448.0f, 448.0f);
+      const float l2 = __builtin_amdgcn_fmed3f((v[2] - bf16_lo(r.hi[1])) * S, -448.0f, 448.0f);
+      const float l3 = __builtin_amdgcn_fmed3f((v[3] - bf16_hi(r.hi[1])) * S, -448.0f, 448.0f);
+      int w = __builtin_amdgcn_cvt_pk_fp8_f32(l0, l1, 0, false);
+      r.lo[0] = __builtin_amdgcn_cvt_pk_fp8_f32(l2, l3, w, true);
+    }
   }
   return r;
 }
@@ -119,6 +131,8 @@ __device__ __forceinline__ void put4(unsigned char *smem, int pbase, int sw, int
     *reinterpret_cast<v2i *>(smem + pbase + (o ^ sw)) = r.hi;
     if constexpr (P::SPLIT)
       *reinterpret_cast<v2i *>(smem + pbase + ((o + Geo<P>::PLANE) ^ sw)) = r.lo;
+    if constexpr (P::LO8)  // one byte per channel: channel index = o / 2
+      *reinterpret_cast<int *>(smem + pbase + Geo<P>::LO_OFF + (o >> 1)) = r.lo[0];
   }
 }
 
@@ -325,6 +339,95 @@ __device__ __forceinline__ void conv3_pass(const unsigned char *smem, const v4i 
   }
 }
 
+// Second pass of the bf16 + fp8 mode over a 3x3 layer: acc += W8 * LO8, both e4m3, K = 64
+// per MFMA.  Lane half h of chunk c contracts half-chunk g = 2c + h = (tap, 32-channel block).
+// A runtime loop over groups of D chunks (D = ring depth) keeps the compiler from hoisting
+// every fragment load of the layer to the front.
+template <class P, int L>
+__device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
+                                              const unsigned char *packed, const float *tail,
+                                              const int (&ci)[3], int h, int lane,
+                                              f32x16 (&acc)[kCoutArr[L] / 32][3]) {
+  using G = Geo<P>;
+  constexpr int NT = kCoutArr[L] / 32, PER32 = kCinArr[L] / 32;
+  constexpr int HC = G::lo_half_chunks(L), NC = G::lo_chunks(L);
+  constexpr int D = (NC % 3 == 0) ? 3 : ((NC % 2 == 0) ? 2 : NC);  // 5 -> 5, 9 -> 3, 14 -> 2
+  static_assert(D <= 5 && NC % D == 0, "fp8 weight ring shape");
+  typedef int v8i __attribute__((ext_vector_type(8)));
+  const v4i *wl = reinterpret_cast<const v4i *>(packed + (size_t)G::lo_frag_offset(L) * 1024) + lane;
+  v4i ring[D][NT][2];
+#pragma unroll
+  for (int d = 0; d < D; ++d)
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int pc = 0; pc < 2; ++pc) ring[d][t][pc] = wl[((d * NT + t) * 2 + pc) * 64];
+  const int sw = reinterpret_cast<const int *>(tail)[G::TAIL_SW + L];
+  const int scale_w = 127 - sw;            // E8M0 exponent undoing the weight copy's 2^sw
+  const int scale_x = 127 - kLoScaleLog2;  // ... and the activations' 2^kLoScaleLog2
+
+  int pbase[3];
+#pragma unroll
+  for (int j = 0; j < 3; ++j) pbase[j] = ci[j] * G::PIXB + G::LO_OFF;
+  // byte offset of this lane half's half-chunk of chunk c, relative to the centre position
+  auto half_off = [&](int c) {
+    int g = 2 * c + h;
+    g = g < HC ? g : HC - 1;  // the padding half-chunk re-reads the last one (its weights are zero)
+    const int tap = g / PER32, cb = g - tap * PER32;
+    const int ky = tap / 3, kx = tap - 3 * ky;
+    return ((ky - 1) * kPitch + (kx - 1)) * G::PIXB + cb * 32;
+  };
+  auto fetch = [&](int c, v4i (&b)[3][2]) {
+    const int off = half_off(c);
+#pragma unroll
+    for (int j = 0; j < 3; ++j) {
+      b[j][0] = *reinterpret_cast<const v4i *>(smem + pbase[j] + off);
+      b[j][1] = *reinterpret_cast<const v4i *>(smem + pbase[j] + off + 16);
+    }
+  };
+  v4i bcur[3][2];
+  fetch(0, bcur);
+#pragma unroll 1
+  for (int c0 = 0; c0 < NC; c0 += D) {
+    const v4i *wn = wl + (size_t)(c0 + D) * NT * 2 * 64;
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      v4i bnext[3][2];
+      fetch(c0 + d + 1 < NC ? c0 + d + 1 : NC - 1, bnext);  // (after the last chunk: a harmless re-read)
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        const v8i a = __builtin_shufflevector(ring[d][t][0], ring[d][t][1], 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+          const v8i b = __builtin_shufflevector(bcur[j][0], bcur[j][1], 0, 1, 2, 3, 4, 5, 6, 7);
+          acc[t][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[t][j], 0, 0, 0, scale_w, 0,
+                                                                      scale_x);
+        }
+      }
+      // weights of chunk c0 + d + D (the tail over-reads the next layer's copy or the zero padding)
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int pc = 0; pc < 2; ++pc) ring[d][t][pc] = wn[((d * NT + t) * 2 + pc) * 64];
+#pragma unroll
+      for (int i = 0; i < NT * 3; ++i) {  // one memory instruction between consecutive MFMAs
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if (i < 6) {
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        } else if (i < 6 + NT * 2) {
+          __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int j = 0; j < 3; ++j) {
+        bcur[j][0] = bnext[j][0];
+        bcur[j][1] = bnext[j][1];
+      }
+    }
+  }
+}
+
 // SiLU of the four accumulators (tile t, pixel tile j, quad q): bias was added at init
 template <class P, int NT>
 __device__ __forceinline__ Packed4<P> silu_quad(const f32x16 (&acc)[NT][3], int t, int j, int q) {
@@ -418,6 +521,7 @@ __device__ __forceinline__ void mid_layer(unsigned char *smem, const unsigned ch
   } else {
     conv3_pass<P, CIN, COUT, 0, 3, false, false>(smem, wl, ring, ci, h, acc, NoSide{});
   }
+  if constexpr (P::LO8) conv3_lo_pass<P, L>(smem, packed, tail, ci, h, lane, acc);
   preload_ring(next, layer_weights<P, L + 1>(packed, lane));
 #ifdef C6_TRACE
   {
@@ -609,6 +713,7 @@ __global__ __launch_bounds__(kThreads) void fused_forward_kernel(const FwdParams
       } else {
         conv3_pass<P, 96, 96, 0, 3, false, false>(smem, wl, r8, ci, h, acc, NoSide{});
       }
+      if constexpr (P::LO8) conv3_lo_pass<P, 7>(smem, packed, tail, ci, h, lane, acc);
       if (bn < prm.total_boards) preload_ring(r1, layer_weights<P, 0>(packed_of(bn), lane));
       C6_MARK(18);
 #pragma unroll
@@ -688,8 +793,36 @@ template <class P> __global__ void pack_kernel(const PackParams prm) {
     unsigned char *dst = prm.packed + (size_t)gid * 16;
     int l = 0;
     while (l < 8 && frag >= G::frag_offset(l + 1)) ++l;  // frag_offset is monotone
-    if (l >= 8) {  // over-read padding
-      *reinterpret_cast<v4i *>(dst) = v4i{0, 0, 0, 0};
+    if (l >= 8) {  // over-read padding, or the fp8 weight copy behind it
+      v4i o = {0, 0, 0, 0};
+      if constexpr (P::LO8) {
+        int ll = 1;
+        while (ll < 8 && frag >= G::lo_frag_offset(ll + 1)) ++ll;
+        if (frag >= G::HI_FRAGS && ll < 8) {
+          const int fi = frag - G::lo_frag_offset(ll);
+          const int cin = kCinArr[ll], nt = kCoutArr[ll] / 32, per32 = cin / 32;
+          const int c = fi / (nt * 2), t = (fi / 2) % nt, piece = fi & 1;
+          const int g = 2 * c + h;
+          if (g < G::lo_half_chunks(ll)) {
+            const int tap = g / per32, cb = g % per32, co = 32 * t + m;
+            const float *w = prm.conv_w[ll];
+            const float sc = exp2f((float)reinterpret_cast<const int *>(prm.packed + G::TAIL_OFF)[G::TAIL_SW + ll]);
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+              float v[4];
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                const int ch = cb * 32 + piece * 16 + d * 4 + e;
+                // the copy approximates the bf16 weights the main pass uses
+                v[e] = __builtin_amdgcn_fmed3f((float)(__bf16)w[(co * cin + ch) * 9 + tap] * sc, -448.0f, 448.0f);
+              }
+              int q = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], 0, false);
+              o[d] = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], q, true);
+            }
+          }
+        }
+      }
+      *reinterpret_cast<v4i *>(dst) = o;
       return;
     }
     const int fi = frag - G::frag_offset(l);
@@ -720,7 +853,7 @@ template <class P> __global__ void pack_kernel(const PackParams prm) {
   }
   // fp32 tail: biases, head weights, head biases
   const int ti = (int)(gid - nfl);
-  if (ti < G::TAIL_FLOATS) {
+  if (ti < G::TAIL_SW) {  // the sw[] words behind it are written by lo_scale_kernel
     float *tail = reinterpret_cast<float *>(prm.packed + G::TAIL_OFF);
     float v = 0.0f;
     if (ti < kBiasTotal) {
@@ -740,6 +873,32 @@ template <class P> __global__ void pack_kernel(const PackParams prm) {
   }
 }
 
+// sw[l] = largest power of two that keeps 2^sw * max|w_l| inside e4m3's range (one block per layer)
+template <class P> __global__ __launch_bounds__(256) void lo_scale_kernel(const PackParams prm) {
+  using G = Geo<P>;
+  __shared__ float red[256];
+  const int l = blockIdx.x;
+  int *sw = reinterpret_cast<int *>(prm.packed + G::TAIL_OFF) + G::TAIL_SW;
+  if (l == 0) {
+    if (threadIdx.x == 0) sw[0] = 0;
+    return;
+  }
+  const int n = kCoutArr[l] * kCinArr[l] * 9;
+  float m = 0.0f;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) m = fmaxf(m, fabsf(prm.conv_w[l][i]));
+  red[threadIdx.x] = m;
+  __syncthreads();
+  for (int s = 128; s > 0; s >>= 1) {
+    if ((int)threadIdx.x < s) red[threadIdx.x] = fmaxf(red[threadIdx.x], red[threadIdx.x + s]);
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    int e = 0;
+    if (red[0] > 0.0f && red[0] < INFINITY) e = (int)floorf(log2f(448.0f / red[0]));
+    sw[l] = e < -20 ? -20 : (e > 20 ? 20 : e);
+  }
+}
+
 // ------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------
@@ -748,6 +907,7 @@ template <class P> static int launch_pack(const PackParams &pp, hipStream_t st) 
   const long long total = (long long)G::TOTAL_FRAGS * 64 + G::TAIL_FLOATS;
   const int threads = 256;
   const int blocks = (int)((total + threads - 1) / threads);
+  if constexpr (P::LO8) hipLaunchKernelGGL(lo_scale_kernel<P>, dim3(8), dim3(256), 0, st, pp);
   hipLaunchKernelGGL(pack_kernel<P>, dim3(blocks), dim3(threads), 0, st, pp);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
@@ -762,8 +922,8 @@ template <class P> static int launch_forward(const FwdParams &fp, hipStream_t st
   static_assert(G::LDS_BYTES <= 160 * 1024, "activation tile must fit the 160 KiB LDS of a CU");
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
-  static thread_local int configured_dev[4] = {-1, -1, -1, -1};
-  static thread_local int cus[4] = {0, 0, 0, 0};
+  static thread_local int configured_dev[5] = {-1, -1, -1, -1, -1};
+  static thread_local int cus[5] = {0, 0, 0, 0, 0};
   if (e == hipSuccess && configured_dev[P::ID] != dev) {
     e = hipFuncSetAttribute(reinterpret_cast<const void *>(&fused_forward_kernel<P>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, G::LDS_BYTES);
@@ -796,6 +956,7 @@ int dispatch_pack(int prec, const PackParams &pp, hipStream_t st) {
     case C6_PREC_BF16: return launch_pack<PrecBF16>(pp, st);
     case C6_PREC_F16: return launch_pack<PrecF16>(pp, st);
     case C6_PREC_BF16X2: return launch_pack<PrecBF16X2>(pp, st);
+    case C6_PREC_BF16F8: return launch_pack<PrecBF16F8>(pp, st);
   }
   set_error("unknown precision mode %d", prec);
   return C6_EINVAL;
@@ -807,6 +968,7 @@ int dispatch_forward(int prec, const FwdParams &fp, hipStream_t st) {
     case C6_PREC_BF16: return launch_forward<PrecBF16>(fp, st);
     case C6_PREC_F16: return launch_forward<PrecF16>(fp, st);
     case C6_PREC_BF16X2: return launch_forward<PrecBF16X2>(fp, st);
+    case C6_PREC_BF16F8: return launch_forward<PrecBF16F8>(fp, st);
   }
   set_error("unknown precision mode %d", prec);
   return C6_EINVAL;
@@ -818,6 +980,7 @@ size_t packed_bytes(int prec) {
     case C6_PREC_BF16: return Geo<PrecBF16>::PACKED_BYTES;
     case C6_PREC_F16: return Geo<PrecF16>::PACKED_BYTES;
     case C6_PREC_BF16X2: return Geo<PrecBF16X2>::PACKED_BYTES;
+    case C6_PREC_BF16F8: return Geo<PrecBF16F8>::PACKED_BYTES;
   }
   return 0;
 }

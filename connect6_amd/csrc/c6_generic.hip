@@ -117,6 +117,7 @@ int launch_generic(const void *x, int x_dtype, long long batch, int n, int layer
                    static_cast<float *>(workspace) + (size_t)batch * cmax * n * n};
   // arithmetic contract of each mode: which operands are rounded to 16 bits
   const int round_w = prec == C6_PREC_F32 ? C6_DT_F32 : (prec == C6_PREC_F16 ? C6_DT_F16 : C6_DT_BF16);
+  // (the hi+lo modes carry the activations' low-order bits: no activation rounding here)
   const int round_a = prec == C6_PREC_BF16 ? C6_DT_BF16 : (prec == C6_PREC_F16 ? C6_DT_F16 : C6_DT_F32);
   const void *in = x;
   int in_dtype = x_dtype;

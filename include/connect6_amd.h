@@ -35,6 +35,8 @@ extern "C" {
 #define C6_PREC_BF16 1   /* bf16 operands, bf16 MFMA, fp32 accumulate, bf16 layer boundaries */
 #define C6_PREC_F16 2    /* fp16 operands, fp16 MFMA, fp32 accumulate, fp16 layer boundaries */
 #define C6_PREC_BF16X2 3 /* bf16 MFMA, activations carried as a bf16 hi+lo pair (two passes)  */
+#define C6_PREC_BF16F8 4 /* bf16 MFMA + a second pass on the activations' dropped low-order
+                            part held as scaled fp8 (e4m3), on the fp8 MFMA at twice the rate */
 
 /* element types of caller tensors */
 #define C6_DT_F32 0

@@ -32,11 +32,16 @@ def test_packed_sizes_follow_the_layout():
         for cin, cout in zip((32, 32, 64, 64, 64, 96, 96), (32, 64, 64, 64, 96, 96, 96)):
             n += (9 * cin // kstep) * (cout // 32)
         return n + 24
-    tail = (544 + 96 + 96 + 4) * 4
+    tail = (544 + 96 + 96 + 4 + 8) * 4
     assert _lib.packed_bytes(_lib.PREC_BF16) == frags(8) * 1024 + tail
     assert _lib.packed_bytes(_lib.PREC_F16) == frags(8) * 1024 + tail
     assert _lib.packed_bytes(_lib.PREC_BF16X2) == frags(8) * 1024 + tail
     assert _lib.packed_bytes(_lib.PREC_F32) == frags(4) * 1024 + tail
+    # bf16 + fp8: plus the e4m3 copy of the 3x3 layers (64-wide chunks, two 16-byte pieces per lane)
+    lo = 0
+    for cin, cout in zip((32, 32, 64, 64, 64, 96, 96), (32, 64, 64, 64, 96, 96, 96)):
+        lo += ((9 * cin // 32 + 1) // 2) * (cout // 32) * 2
+    assert _lib.packed_bytes(_lib.PREC_BF16F8) == (frags(8) + lo + 18) * 1024 + tail
     with pytest.raises(ValueError):
         _lib.packed_bytes(9)
 
