@@ -108,14 +108,19 @@ template <class P> __device__ __forceinline__ Packed4<P> pack4(const float (&v)[
       r.lo[0] = pack2<P>(v[0] - bf16_lo(r.hi[0]), v[1] - bf16_hi(r.hi[0]));
       r.lo[1] = pack2<P>(v[2] - bf16_lo(r.hi[1]), v[3] - bf16_hi(r.hi[1]));
     }
-    if constexpr (P::LO8) {  // dropped low-order parts, scaled, as four e4m3 bytes
-      constexpr float S = (float)(1 << kLoScaleLog2);
-      const float l0 = __builtin_amdgcn_fmed3f((v[0] - bf16_lo(r.hi[0])) * S, -448.0f, 448.0f);
-      const float l1 = __builtin_amdgcn_fmed3f((v[1] - bf16_hi(r.hi[0])) * S, -448.0f, 448.0f);
-      const float l2 = __builtin_amdgcn_fmed3f((v[2] - bf16_lo(r.hi[1])) * S, -448.0f, 448.0f);
-      const float l3 = __builtin_amdgcn_fmed3f((v[3] - bf16_hi(r.hi[1])) * S, -448.0f, 448.0f);
-      int w = __builtin_amdgcn_cvt_pk_fp8_f32(l0, l1, 0, false);
-      r.lo[0] = __builtin_amdgcn_cvt_pk_fp8_f32(l2, l3, w, true);
+    if constexpr (P::LO8) {  // dropped low-order parts as four e4m3 bytes of lo * 2^kLoScaleLog2
+      // v_cvt_scalef32_pk_fp8_f32 divides by its scale operand and turns overflow into NaN,
+      // so the inputs are clamped to what 448 * 2^-kLoScaleLog2 can represent.
+      constexpr float INV = 1.0f / (float)(1 << kLoScaleLog2), LIM = 448.0f * INV;
+      typedef short v2s __attribute__((ext_vector_type(2)));
+      const float l0 = __builtin_amdgcn_fmed3f(v[0] - bf16_lo(r.hi[0]), -LIM, LIM);
+      const float l1 = __builtin_amdgcn_fmed3f(v[1] - bf16_hi(r.hi[0]), -LIM, LIM);
+      const float l2 = __builtin_amdgcn_fmed3f(v[2] - bf16_lo(r.hi[1]), -LIM, LIM);
+      const float l3 = __builtin_amdgcn_fmed3f(v[3] - bf16_hi(r.hi[1]), -LIM, LIM);
+      v2s w = {0, 0};
+      w = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(w, l0, l1, INV, false);
+      w = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(w, l2, l3, INV, true);
+      r.lo[0] = __builtin_bit_cast(int, w);
     }
   }
   return r;
