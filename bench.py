@@ -176,6 +176,15 @@ def main() -> int:
         ts = timed(lambda: model.selfplay_step(xs, us, 1.0), steps=10)
         out["selfplay_step_b16384"] = {"boards_per_s": 16384 / ts, "ms": ts * 1e3}
 
+        # ---- the same step fed from int8 environment state (view + canonical input + gather in the loader) ----
+        occ_ = (xs[:, 0] + xs[:, 1]) > 0
+        boards8 = (xs[:, 0] - xs[:, 1]).to(torch.int8)
+        player8 = torch.ones(16384, dtype=torch.int8, device=dev)
+        left8 = torch.ones(16384, dtype=torch.int8, device=dev)
+        tsb = timed(lambda: model.selfplay_step_boards(boards8, player8, left8, us, 1.0, view=5), steps=10)
+        out["selfplay_step_from_int8_boards_b16384"] = {"boards_per_s": 16384 / tsb, "ms": tsb * 1e3}
+        del occ_
+
         # ---- D4-averaged evaluation, configs[4]: 8192 base boards -> 65536 views ----
         xd = gen_boards(8192, 200, 2025)[0].to(dev)
         td = timed(lambda: c6.evaluate_d4(model, xd), steps=5, warmup=2)

@@ -30,6 +30,7 @@ EXPORTS = (
     "c6_packed_bytes",
     "c6_pack_weights",
     "c6_forward",
+    "c6_forward_boards",
     "c6_generic_workspace_bytes",
     "c6_forward_generic",
     "c6_mask_logits",
@@ -88,6 +89,9 @@ def load() -> ctypes.CDLL:
     lib.c6_forward.restype = i32
     lib.c6_forward.argtypes = [vp, i32, i64, i64, vp, ctypes.c_size_t, i32, vp, vp, i32, vp, f32,
                                vp, f32, vp, vp, vp]
+    lib.c6_forward_boards.restype = i32
+    lib.c6_forward_boards.argtypes = [vp, vp, vp, vp, i32, i64, vp, i32, vp, vp, i32, f32, vp, f32,
+                                      vp, vp, vp]
     ip = ctypes.POINTER(ctypes.c_int)
     lib.c6_generic_workspace_bytes.restype = i32
     lib.c6_generic_workspace_bytes.argtypes = [i64, i32, i32, ip, ctypes.POINTER(ctypes.c_size_t)]

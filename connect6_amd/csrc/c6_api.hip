@@ -144,6 +144,58 @@ int c6_forward(const void *x, int x_dtype, int64_t groups, int64_t boards_per_gr
   fp.inv_temperature = 1.0f / (temperature > 1e-4f ? temperature : 1e-4f);
   fp.actions = reinterpret_cast<long long *>(actions);
   fp.logprob = logprob;
+  fp.player = nullptr;
+  fp.stones_left = nullptr;
+  fp.index = nullptr;
+  fp.view = 0;
+  return dispatch_forward(prec, fp, static_cast<hipStream_t>(stream));
+}
+
+int c6_forward_boards(const int8_t *boards, const int8_t *player, const int8_t *stones_left,
+                      const int64_t *index, int view, int64_t batch, const void *packed, int prec,
+                      float *logits, float *value, int mask_mode, float fill, const float *u,
+                      float temperature, int64_t *actions, float *logprob, void *stream) {
+  if (!valid_prec(prec) || batch < 0 || batch > 0x7fffffffLL || view < 0 || view > 7) {
+    set_error("c6_forward_boards: bad precision %d, batch %lld or view %d", prec, (long long)batch, view);
+    return C6_EINVAL;
+  }
+  if (batch == 0) return C6_OK;
+  if (boards == nullptr || player == nullptr || stones_left == nullptr || packed == nullptr) {
+    set_error("c6_forward_boards: boards, player, stones_left and packed must not be null");
+    return C6_EINVAL;
+  }
+  if (!aligned16(packed)) {
+    set_error("c6_forward_boards: packed weights must be 16-byte aligned");
+    return C6_EINVAL;
+  }
+  if (mask_mode != C6_MASK_NONE && mask_mode != C6_MASK_INPUT) {
+    set_error("c6_forward_boards: mask_mode must be C6_MASK_NONE or C6_MASK_INPUT, got %d", mask_mode);
+    return C6_EINVAL;
+  }
+  if (actions != nullptr && u == nullptr) {
+    set_error("c6_forward_boards: sampling needs the uniform draws u");
+    return C6_EINVAL;
+  }
+  FwdParams fp;
+  fp.x = boards;
+  fp.x_dtype = C6_DT_BOARD_I8;
+  fp.total_boards = batch;
+  fp.boards_per_group = batch;
+  fp.packed = static_cast<const unsigned char *>(packed);
+  fp.packed_stride = 0;
+  fp.logits = logits;
+  fp.value = value;
+  fp.mask_mode = mask_mode;
+  fp.legal = nullptr;
+  fp.fill = fill;
+  fp.u = u;
+  fp.inv_temperature = 1.0f / (temperature > 1e-4f ? temperature : 1e-4f);
+  fp.actions = reinterpret_cast<long long *>(actions);
+  fp.logprob = logprob;
+  fp.player = player;
+  fp.stones_left = stones_left;
+  fp.index = reinterpret_cast<const long long *>(index);
+  fp.view = view;
   return dispatch_forward(prec, fp, static_cast<hipStream_t>(stream));
 }
 

@@ -169,6 +169,11 @@ struct FwdParams {
   float inv_temperature;
   long long *actions;
   float *logprob;
+  // board-state input (x_dtype == C6_DT_BOARD_I8): x is int8 boards [N,19,19] with +1/-1/0
+  const int8_t *player;       // [N] side to move (+1 / -1)
+  const int8_t *stones_left;  // [N] stones left in the turn
+  const long long *index;     // [B] rows of the state tensors to evaluate, or null for 0..B-1
+  int view;                   // D4 view 0..7 applied to the board before evaluation
 };
 
 struct PackParams {

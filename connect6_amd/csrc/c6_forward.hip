@@ -584,6 +584,26 @@ __global__ __launch_bounds__(kThreads) void fused_forward_kernel(const FwdParams
   float xin[2][3];
   unsigned char occin[2];
   auto fetch_board = [&](long long b) {
+    if (prm.x_dtype == C6_DT_BOARD_I8) {
+      // environment state in, network planes out (connect6/vector_env.py:196-218 of the
+      // reference), seen through D4 view prm.view (connect6/train.py:222-230)
+      const long long src = prm.index ? prm.index[b] : b;
+      const int8_t *board = reinterpret_cast<const int8_t *>(prm.x) + (size_t)src * kPix;
+      const int me = prm.player[src];
+      const float last = prm.stones_left[src] == 1 ? 1.0f : 0.0f;
+#pragma unroll
+      for (int r = 0; r < 2; ++r) {
+        const int p = tid + r * kThreads;
+        if (p < kPix) {
+          const int stone = board[prm.view ? d4_from_view(p, prm.view) : p];
+          xin[r][0] = stone == me ? 1.0f : 0.0f;
+          xin[r][1] = stone == -me ? 1.0f : 0.0f;
+          xin[r][2] = last;
+          occin[r] = 0;
+        }
+      }
+      return;
+    }
 #pragma unroll
     for (int r = 0; r < 2; ++r) {
       const int p = tid + r * kThreads;

@@ -398,6 +398,121 @@ class PolicyValueNet(nn.Module):
             return actions, logprob, value, logits
         return actions, logprob, value
 
+    def forward_boards(
+        self,
+        boards: torch.Tensor,
+        current_player: torch.Tensor,
+        stones_left: torch.Tensor,
+        *,
+        index: torch.Tensor | None = None,
+        view: int = 0,
+        masked: bool = True,
+        fill: float | None = None,
+    ) -> tuple[torch.Tensor, torch.Tensor]:
+        """Forward straight from the environment's int8 state
+        (``VectorConnect6.boards / .current_player / .stones_left``): one launch
+        does what the reference's collector does per step with
+        ``_transform_boards`` (D4 ``view`` 0..7, connect6/train.py:730-741),
+        ``canonical_network_input`` (connect6/vector_env.py:196-218), the row
+        gather ``network_input[index]``, the forward and -- with ``masked`` --
+        ``mask_logits(logits.float(), view_boards == 0)``.  Logits are in view
+        coordinates, as in the reference."""
+        logits, value, _, _ = _forward_boards(self, boards, current_player, stones_left, index=index,
+                                              view=view, masked=masked, fill=fill, u=None,
+                                              temperature=1.0, want_logits=True)
+        return logits, value
+
+    def selfplay_step_boards(
+        self,
+        boards: torch.Tensor,
+        current_player: torch.Tensor,
+        stones_left: torch.Tensor,
+        u: torch.Tensor,
+        temperature: float = 1.0,
+        *,
+        index: torch.Tensor | None = None,
+        view: int = 0,
+    ):
+        """``forward_boards`` + masked softmax + one inverse-CDF draw per board
+        (``_sample_actions``, connect6/train.py:195-203) in the same launch.
+        Returns ``(actions, logprob, value)``; actions are in view coordinates
+        (map them back with ``inverse_transform_actions``)."""
+        _, value, actions, logprob = _forward_boards(self, boards, current_player, stones_left,
+                                                     index=index, view=view, masked=True, fill=None,
+                                                     u=u, temperature=temperature, want_logits=False)
+        return actions, logprob, value
+
+
+def _state_tensor(t: torch.Tensor, name: str, shape, dev) -> torch.Tensor:
+    if t.dtype != torch.int8:
+        raise ValueError(f"{name} must be an int8 tensor (as VectorConnect6 holds it), got {t.dtype}")
+    if tuple(t.shape) != tuple(shape):
+        raise ValueError(f"{name} must have shape {tuple(shape)}, got {tuple(t.shape)}")
+    return t.to(dev).contiguous()
+
+
+def _forward_boards(
+    model: "PolicyValueNet",
+    boards: torch.Tensor,
+    current_player: torch.Tensor,
+    stones_left: torch.Tensor,
+    *,
+    index: torch.Tensor | None,
+    view: int,
+    masked: bool,
+    fill: float | None,
+    u: torch.Tensor | None,
+    temperature: float,
+    want_logits: bool,
+):
+    _require_device_tensor(boards, "boards")
+    _require_device_tensor(model.convs[0].weight, "model parameters")
+    if not model.is_default_architecture:
+        raise NotImplementedError("board-state input is built for the default architecture on a 19x19 board")
+    if torch.is_grad_enabled() and any(p.requires_grad for p in model.parameters()):
+        raise RuntimeError("connect6_amd.PolicyValueNet is the inference forward only: call it under "
+                           "torch.no_grad() / torch.inference_mode()")
+    if boards.ndim != 3 or tuple(boards.shape[1:]) != (19, 19):
+        raise ValueError(f"boards must have shape [N, 19, 19], got {tuple(boards.shape)}")
+    if not 0 <= int(view) <= 7:
+        raise ValueError(f"view must be a D4 phase 0..7, got {view}")
+    dev = boards.device
+    n = int(boards.shape[0])
+    boards = _state_tensor(boards, "boards", (n, 19, 19), dev)
+    current_player = _state_tensor(current_player, "current_player", (n,), dev)
+    stones_left = _state_tensor(stones_left, "stones_left", (n,), dev)
+    if index is not None:
+        if index.dtype != torch.int64 or index.ndim != 1:
+            raise ValueError("index must be a 1-D int64 tensor of board rows")
+        index = index.to(dev).contiguous()
+        if index.numel() and (int(index.min()) < 0 or int(index.max()) >= n):
+            raise ValueError(f"index entries must lie in [0, {n})")
+    b = n if index is None else int(index.numel())
+    prec = model.resolve_precision()
+    packed = model.packed_weights(prec)
+    logits = torch.empty((b, 361), dtype=torch.float32, device=dev) if want_logits else None
+    value = torch.empty((b,), dtype=torch.float32, device=dev)
+    actions = logprob = None
+    if u is not None:
+        u = u.to(device=dev, dtype=torch.float32).contiguous()
+        if u.shape != (b,):
+            raise ValueError(f"u must have shape ({b},), got {tuple(u.shape)}")
+        actions = torch.empty((b,), dtype=torch.int64, device=dev)
+        logprob = torch.empty((b,), dtype=torch.float32, device=dev)
+
+    def ptr(t):
+        return t.data_ptr() if t is not None else None
+
+    with torch.cuda.device(dev):
+        rc = _lib.load().c6_forward_boards(
+            boards.data_ptr(), current_player.data_ptr(), stones_left.data_ptr(), ptr(index),
+            int(view), b, packed.data_ptr(), prec, ptr(logits), value.data_ptr(),
+            _lib.MASK_INPUT if masked else _lib.MASK_NONE,
+            _FILL_LOWEST if fill is None else float(fill), ptr(u), float(temperature),
+            ptr(actions), ptr(logprob), _lib.stream_ptr(dev))
+    _lib.check(rc, "c6_forward_boards")
+    return logits, value, actions, logprob
+
 
 def build_model(model_cfg: dict[str, Any], board_size: int) -> PolicyValueNet:
     """Build the CNN from the ``model`` section of the YAML config

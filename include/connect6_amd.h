@@ -42,6 +42,7 @@ extern "C" {
 #define C6_DT_F32 0
 #define C6_DT_BF16 1
 #define C6_DT_F16 2
+#define C6_DT_BOARD_I8 3 /* int8 board states (+1 / -1 / 0), only through c6_forward_boards */
 
 /* masking of occupied squares in the policy logits */
 #define C6_MASK_NONE 0   /* logits as the network produced them (PolicyValueNet.forward)    */
@@ -88,6 +89,25 @@ int c6_forward(const void *x, int x_dtype, int64_t groups, int64_t boards_per_gr
                float *value, int mask_mode, const uint8_t *legal, float fill,
                const float *u, float temperature, int64_t *actions, float *logprob,
                void *stream);
+
+/* The same forward, fed directly from the environment's state tensors instead of float planes.
+ * Replaces, in one launch, the collector's per-step chain (connect6/train.py:730-748,
+ * :791-799): _transform_boards(boards, view) -> canonical_network_input (connect6/
+ * vector_env.py:196-218: plane 0 = boards == player, plane 1 = boards == -player, plane 2 =
+ * stones_left == 1) -> optional row gather (network_input[index]) -> forward -> mask_logits
+ * with legal = view_boards == 0 -> optional sampling.
+ *   boards       device int8 [N,19,19], values +1 / -1 / 0
+ *   player       device int8 [N], side to move (+1 / -1)
+ *   stones_left  device int8 [N]
+ *   index        device int64 [B] rows of the state tensors to evaluate, or NULL (B = N rows 0..B-1)
+ *   view         D4 view 0..7 (numbering of _symmetry_for_phase); outputs are in view coordinates
+ *   mask_mode    C6_MASK_NONE or C6_MASK_INPUT (occupied squares of the viewed board)
+ * Remaining arguments as c6_forward with groups = 1. */
+int c6_forward_boards(const int8_t *boards, const int8_t *player, const int8_t *stones_left,
+                      const int64_t *index, int view, int64_t batch, const void *packed,
+                      int prec, float *logits, float *value, int mask_mode, float fill,
+                      const float *u, float temperature, int64_t *actions, float *logprob,
+                      void *stream);
 
 /* Forward of ONE weight set for any architecture the reference's PolicyValueNet accepts
  * (connect6/model.py:26-77: any board size, odd kernels, positive channel counts), layer by

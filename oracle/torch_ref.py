@@ -24,6 +24,8 @@ function               pinned by (tests/test_oracle.py)
                        single(model_i, x[i]) (tests/test_training_features.py
                        :120-151 of the reference).
 ``mask_logits``        closed form; bit-pattern check of fill / untouched.
+``canonical_network_   channel meaning as the reference tests it (tests/test_game.py
+input``                :46-59, :62-75): hand-built position, values exactly {0,1}.
 ``sample_inverse_cdf`` brute-force python loop on tiny inputs; empirical
                        distribution vs softmax; never picks a masked square.
 ``transform_*``        the reference's property tests (tests/test_model.py
@@ -228,6 +230,18 @@ def sample_inverse_cdf(
     a = torch.minimum(a, last_legal)
     logp = z.gather(1, a.view(-1, 1)).squeeze(1) - zmax.squeeze(1) - torch.log(total.squeeze(1))
     return a, logp
+
+
+def canonical_network_input(boards: torch.Tensor, current_player: torch.Tensor,
+                            stones_left: torch.Tensor) -> torch.Tensor:
+    """connect6/vector_env.py:196-218: int8 boards [N,n,n] (+1/-1/0), side to move [N],
+    stones left [N] -> fp32 planes [N,3,n,n]: own stones, opponent stones, "last stone of
+    the turn" flag broadcast over the board."""
+    player = current_player.view(-1, 1, 1)
+    me = boards.eq(player).to(torch.float32)
+    opp = boards.eq(-player).to(torch.float32)
+    last = stones_left.eq(1).to(torch.float32).view(-1, 1, 1).expand(-1, boards.shape[-2], boards.shape[-1])
+    return torch.stack((me, opp, last), dim=1)
 
 
 # --------------------------------------------------------------------------

@@ -147,3 +147,64 @@ def test_d4_evaluation_cfg5(cuda):
     a = torch.arange(361, device=cuda)
     back = rot_l[:, c6.transform_actions(a, 19, k, flip)]
     assert torch.allclose(back, base_l, atol=1e-6) and torch.allclose(rot_v, base_v, atol=1e-6)
+
+
+def _random_states(n, seed):
+    g = torch.Generator().manual_seed(seed)
+    x, _ = gen_boards(n, 250, seed)
+    player = (torch.randint(0, 2, (n,), generator=g) * 2 - 1).to(torch.int8)
+    # planes are side-to-move relative; rebuild absolute colours
+    boards = ((x[:, 0] - x[:, 1]) * player.view(-1, 1, 1).float()).to(torch.int8)
+    left = torch.randint(1, 3, (n,), generator=g).to(torch.int8)
+    return boards, player, left
+
+
+@pytest.mark.parametrize("view", [0, 3, 6])
+def test_forward_from_board_states(cuda, view):
+    """Collector step from the environment's int8 state: view, canonical input, gather, forward, mask."""
+    st = R.init_state(1234, "reference")
+    model = c6.PolicyValueNet().to(cuda).eval()
+    model.load_state_dict(st)
+    boards, player, left = _random_states(300, 5)
+    index = torch.randperm(300, generator=torch.Generator().manual_seed(1))[:200]
+    k, flip = R.symmetry_for_phase(view)
+    view_boards = R.transform_boards(boards, k, flip)               # train.py:730-741
+    x = R.canonical_network_input(view_boards, player, left)        # train.py:743-747
+    legal = view_boards.reshape(300, -1).eq(0)                      # train.py:748
+    with torch.inference_mode():
+        lo, vo = R.forward(st, x[index])                            # train.py:791-794
+        lg, vg = model.forward_boards(boards.to(cuda), player.to(cuda), left.to(cuda),
+                                      index=index.to(cuda), view=view)
+        plain, _ = model.forward_boards(boards.to(cuda), player.to(cuda), left.to(cuda),
+                                        index=index.to(cuda), view=view, masked=False)
+        same, vsame = model.forward_masked(x[index].to(cuda))      # float-plane entry point, same kernel
+    assert rel_l2(plain, lo) <= 1e-4 and rel_l2(vg, vo) <= 1e-4
+    assert torch.equal(lg.cpu(), R.mask_logits(plain.cpu(), legal[index]))   # bit-exact masking
+    assert torch.equal(lg, same) and torch.equal(vg, vsame)
+    # whole batch, no gather, with the fused draw
+    u = gen_uniform(300, 2)
+    model.precision = "bf16f8"
+    with torch.inference_mode():
+        a, lp, v = model.selfplay_step_boards(boards.to(cuda), player.to(cuda), left.to(cuda), u.to(cuda),
+                                              0.9, view=view)
+        a2, lp2, v2 = model.selfplay_step(x.to(cuda), u.to(cuda), 0.9)
+    assert torch.equal(a, a2) and torch.equal(lp, lp2) and torch.equal(v, v2)
+    assert bool(legal.gather(1, a.cpu().view(-1, 1)).all())
+    back = c6.inverse_transform_actions(a.cpu(), 19, k, flip)       # train.py:854-862
+    assert bool((boards.reshape(300, -1).gather(1, back.view(-1, 1)) == 0).all())
+
+
+def test_forward_boards_argument_checks(cuda):
+    model = c6.PolicyValueNet().to(cuda).eval()
+    boards, player, left = (t.to(cuda) for t in _random_states(4, 1))
+    with torch.inference_mode():
+        with pytest.raises(ValueError):
+            model.forward_boards(boards.float(), player, left)
+        with pytest.raises(ValueError):
+            model.forward_boards(boards, player[:3], left)
+        with pytest.raises(ValueError):
+            model.forward_boards(boards, player, left, view=8)
+        with pytest.raises(ValueError):
+            model.forward_boards(boards, player, left, index=torch.tensor([0, 4], device=cuda))
+        logits, value = model.forward_boards(boards, player, left, index=torch.zeros(0, dtype=torch.int64, device=cuda))
+        assert logits.shape == (0, 361) and value.shape == (0,)

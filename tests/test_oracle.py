@@ -242,3 +242,22 @@ def test_generator_properties():
     assert torch.equal(x, x2)
     x3, _ = gen_boards(64, 300, 1)
     assert int((x3[:, 0] + x3[:, 1]).flatten(1).sum(1).max()) > 200
+
+
+def test_canonical_network_input_channel_meaning():
+    # tests/test_game.py:46-59 of the reference: plane 0 = side to move, plane 1 = opponent,
+    # plane 2 = "this is the last stone of the turn"
+    boards = torch.zeros(2, 19, 19, dtype=torch.int8)
+    boards[0, 9, 9] = 1
+    boards[0, 3, 4] = -1
+    boards[1, 0, 0] = -1
+    boards[1, 18, 18] = 1
+    player = torch.tensor([1, -1], dtype=torch.int8)
+    left = torch.tensor([1, 2], dtype=torch.int8)
+    x = R.canonical_network_input(boards, player, left)
+    assert x.shape == (2, 3, 19, 19) and x.dtype == torch.float32
+    assert x[0, 0, 9, 9] == 1 and x[0, 0].sum() == 1
+    assert x[0, 1, 3, 4] == 1 and x[0, 1].sum() == 1
+    assert torch.all(x[0, 2] == 1) and torch.all(x[1, 2] == 0)
+    assert x[1, 0, 0, 0] == 1 and x[1, 1, 18, 18] == 1          # colours swap with the side to move
+    assert torch.equal(R.legal_from_input(x), boards.view(2, -1).eq(0))   # vector_env.py:95-96
