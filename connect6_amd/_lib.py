@@ -90,7 +90,7 @@ def load() -> ctypes.CDLL:
     lib.c6_forward.argtypes = [vp, i32, i64, i64, vp, ctypes.c_size_t, i32, vp, vp, i32, vp, f32,
                                vp, f32, vp, vp, vp]
     lib.c6_forward_boards.restype = i32
-    lib.c6_forward_boards.argtypes = [vp, vp, vp, vp, i32, i64, vp, i32, vp, vp, i32, f32, vp, f32,
+    lib.c6_forward_boards.argtypes = [vp, vp, vp, i64, vp, i32, i64, vp, i32, vp, vp, i32, f32, vp, f32,
                                       vp, vp, vp]
     ip = ctypes.POINTER(ctypes.c_int)
     lib.c6_generic_workspace_bytes.restype = i32

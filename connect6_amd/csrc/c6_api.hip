@@ -147,19 +147,27 @@ int c6_forward(const void *x, int x_dtype, int64_t groups, int64_t boards_per_gr
   fp.player = nullptr;
   fp.stones_left = nullptr;
   fp.index = nullptr;
+  fp.num_states = 0;
   fp.view = 0;
   return dispatch_forward(prec, fp, static_cast<hipStream_t>(stream));
 }
 
 int c6_forward_boards(const int8_t *boards, const int8_t *player, const int8_t *stones_left,
-                      const int64_t *index, int view, int64_t batch, const void *packed, int prec,
+                      int64_t num_states, const int64_t *index, int view, int64_t batch,
+                      const void *packed, int prec,
                       float *logits, float *value, int mask_mode, float fill, const float *u,
                       float temperature, int64_t *actions, float *logprob, void *stream) {
-  if (!valid_prec(prec) || batch < 0 || batch > 0x7fffffffLL || view < 0 || view > 7) {
-    set_error("c6_forward_boards: bad precision %d, batch %lld or view %d", prec, (long long)batch, view);
+  if (!valid_prec(prec) || batch < 0 || batch > 0x7fffffffLL || view < 0 || view > 7 || num_states < 0) {
+    set_error("c6_forward_boards: bad precision %d, batch %lld, states %lld or view %d", prec,
+              (long long)batch, (long long)num_states, view);
     return C6_EINVAL;
   }
   if (batch == 0) return C6_OK;
+  if (num_states < 1 || (index == nullptr && batch > num_states)) {
+    set_error("c6_forward_boards: %lld boards requested from %lld states", (long long)batch,
+              (long long)num_states);
+    return C6_EINVAL;
+  }
   if (boards == nullptr || player == nullptr || stones_left == nullptr || packed == nullptr) {
     set_error("c6_forward_boards: boards, player, stones_left and packed must not be null");
     return C6_EINVAL;
@@ -195,6 +203,7 @@ int c6_forward_boards(const int8_t *boards, const int8_t *player, const int8_t *
   fp.player = player;
   fp.stones_left = stones_left;
   fp.index = reinterpret_cast<const long long *>(index);
+  fp.num_states = num_states;
   fp.view = view;
   return dispatch_forward(prec, fp, static_cast<hipStream_t>(stream));
 }

@@ -173,6 +173,7 @@ struct FwdParams {
   const int8_t *player;       // [N] side to move (+1 / -1)
   const int8_t *stones_left;  // [N] stones left in the turn
   const long long *index;     // [B] rows of the state tensors to evaluate, or null for 0..B-1
+  long long num_states;       // N: index entries are clamped into [0, N) (no out-of-bounds read)
   int view;                   // D4 view 0..7 applied to the board before evaluation
 };
 

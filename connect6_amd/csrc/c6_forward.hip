@@ -587,7 +587,8 @@ __global__ __launch_bounds__(kThreads) void fused_forward_kernel(const FwdParams
     if (prm.x_dtype == C6_DT_BOARD_I8) {
       // environment state in, network planes out (connect6/vector_env.py:196-218 of the
       // reference), seen through D4 view prm.view (connect6/train.py:222-230)
-      const long long src = prm.index ? prm.index[b] : b;
+      long long src = prm.index ? prm.index[b] : b;
+      src = src < 0 ? 0 : (src >= prm.num_states ? prm.num_states - 1 : src);
       const int8_t *board = reinterpret_cast<const int8_t *>(prm.x) + (size_t)src * kPix;
       const int me = prm.player[src];
       const float last = prm.stones_left[src] == 1 ? 1.0f : 0.0f;

@@ -484,9 +484,7 @@ def _forward_boards(
     if index is not None:
         if index.dtype != torch.int64 or index.ndim != 1:
             raise ValueError("index must be a 1-D int64 tensor of board rows")
-        index = index.to(dev).contiguous()
-        if index.numel() and (int(index.min()) < 0 or int(index.max()) >= n):
-            raise ValueError(f"index entries must lie in [0, {n})")
+        index = index.to(dev).contiguous()   # entries outside [0, N) are clamped by the kernel
     b = n if index is None else int(index.numel())
     prec = model.resolve_precision()
     packed = model.packed_weights(prec)
@@ -505,7 +503,7 @@ def _forward_boards(
 
     with torch.cuda.device(dev):
         rc = _lib.load().c6_forward_boards(
-            boards.data_ptr(), current_player.data_ptr(), stones_left.data_ptr(), ptr(index),
+            boards.data_ptr(), current_player.data_ptr(), stones_left.data_ptr(), n, ptr(index),
             int(view), b, packed.data_ptr(), prec, ptr(logits), value.data_ptr(),
             _lib.MASK_INPUT if masked else _lib.MASK_NONE,
             _FILL_LOWEST if fill is None else float(fill), ptr(u), float(temperature),

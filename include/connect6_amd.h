@@ -99,12 +99,15 @@ int c6_forward(const void *x, int x_dtype, int64_t groups, int64_t boards_per_gr
  *   boards       device int8 [N,19,19], values +1 / -1 / 0
  *   player       device int8 [N], side to move (+1 / -1)
  *   stones_left  device int8 [N]
- *   index        device int64 [B] rows of the state tensors to evaluate, or NULL (B = N rows 0..B-1)
+ *   num_states   N
+ *   index        device int64 [B] rows of the state tensors to evaluate (entries outside [0,N)
+ *                are clamped into range), or NULL (rows 0..B-1, B <= N)
  *   view         D4 view 0..7 (numbering of _symmetry_for_phase); outputs are in view coordinates
  *   mask_mode    C6_MASK_NONE or C6_MASK_INPUT (occupied squares of the viewed board)
  * Remaining arguments as c6_forward with groups = 1. */
 int c6_forward_boards(const int8_t *boards, const int8_t *player, const int8_t *stones_left,
-                      const int64_t *index, int view, int64_t batch, const void *packed,
+                      int64_t num_states, const int64_t *index, int view, int64_t batch,
+                      const void *packed,
                       int prec, float *logits, float *value, int mask_mode, float fill,
                       const float *u, float temperature, int64_t *actions, float *logprob,
                       void *stream);

@@ -204,7 +204,9 @@ def test_forward_boards_argument_checks(cuda):
             model.forward_boards(boards, player[:3], left)
         with pytest.raises(ValueError):
             model.forward_boards(boards, player, left, view=8)
-        with pytest.raises(ValueError):
-            model.forward_boards(boards, player, left, index=torch.tensor([0, 4], device=cuda))
+        # rows outside [0, N) are clamped into range by the kernel (never read out of bounds)
+        lc, _ = model.forward_boards(boards, player, left, index=torch.tensor([-3, 9], device=cuda))
+        le, _ = model.forward_boards(boards, player, left, index=torch.tensor([0, 3], device=cuda))
+        assert torch.equal(lc, le)
         logits, value = model.forward_boards(boards, player, left, index=torch.zeros(0, dtype=torch.int64, device=cuda))
         assert logits.shape == (0, 361) and value.shape == (0,)

@@ -61,11 +61,11 @@ def test_entry_points_reject_bad_arguments_before_touching_the_device():
     assert lib.c6_d4_expand(None, 0, 2, None, None) == -1
     assert lib.c6_d4_reduce(None, None, 2, None, None, None) == -1
     assert lib.c6_pack_weights(None, None, None, None, None, None, 1, None, None) == -1
-    assert lib.c6_forward_boards(None, None, None, None, 0, 4, None, 1, None, None, 1, 0.0, None, 1.0,
+    assert lib.c6_forward_boards(None, None, None, 4, None, 0, 4, None, 1, None, None, 1, 0.0, None, 1.0,
                                  None, None, None) == -1
-    assert lib.c6_forward_boards(None, None, None, None, 9, 4, None, 1, None, None, 1, 0.0, None, 1.0,
+    assert lib.c6_forward_boards(None, None, None, 4, None, 9, 4, None, 1, None, None, 1, 0.0, None, 1.0,
                                  None, None, None) == -1
-    assert lib.c6_forward_boards(None, None, None, None, 0, 0, None, 1, None, None, 1, 0.0, None, 1.0,
+    assert lib.c6_forward_boards(None, None, None, 4, None, 0, 0, None, 1, None, None, 1, 0.0, None, 1.0,
                                  None, None, None) == 0
     n = ctypes.c_size_t(0)
     ch = (ctypes.c_int * 3)(8, 8, 16)
