@@ -169,6 +169,16 @@ def main() -> int:
             "workload": f"configs[2]: 8 weight sets x {B // 8} boards, one launch, bf16 in/out",
         }
 
+        # production shape of the history path (configs/train.yaml of the reference: up to 128
+        # frozen models sharing 512 tables): weight traffic per board is 32x the G=8 case
+        cps128 = [cps[i % 8] for i in range(128)]
+        ens128 = c6.HistoricalPolicyEnsemble(cps128, dev, dtype=torch.bfloat16,
+                                             precision=None if args.precision == "fp32" else args.precision)
+        xg128 = x[:512].view(128, 4, 3, 19, 19).to(torch.bfloat16)
+        tg128 = timed(lambda: ens128.forward_grouped(xg128))
+        out["grouped_g128x4"] = {"boards_per_s": 512 / tg128, "ms": tg128 * 1e3}
+        del ens128, cps128
+
         # ---- fused self-play step, configs[3]: B=16384, stones 0..300 ----
         model.precision = args.precision
         xs = gen_boards(16384, 300, 2025)[0].to(dev)

@@ -229,3 +229,20 @@ def test_grouped_g8_bf16_cfg3(cuda, precision):
             st = {k: v.to(torch.bfloat16).float() for k, v in cp.model_state.items()}
             expected, _ = R.forward(st, xg[i])
             assert rel_l2(grouped[i].float(), expected) <= BF16_TOL
+
+
+def test_fp32_matches_committed_golden_vectors(cuda):
+    import numpy as np
+    from pathlib import Path
+
+    g = np.load(Path(__file__).resolve().parent / "golden" / "default_arch_golden.npz")
+    x = torch.from_numpy(g["x"])
+    for init in ("reference", "torch_default"):
+        model = make_model(cuda, R.init_state(1234, init))
+        with torch.inference_mode():
+            logits, value = model(x.to(cuda))
+            actions, logprob, _ = model.selfplay_step(x.to(cuda), torch.from_numpy(g["u"]).to(cuda), 1.0)
+        assert rel_l2(logits, torch.from_numpy(g[f"{init}_logits"])) <= FP32_TOL
+        assert rel_l2(value, torch.from_numpy(g[f"{init}_value"])) <= FP32_TOL
+        assert np.array_equal(actions.cpu().numpy(), g[f"{init}_actions"])
+        assert np.allclose(logprob.cpu().numpy(), g[f"{init}_logprob"], atol=2e-4)

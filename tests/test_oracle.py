@@ -261,3 +261,18 @@ def test_canonical_network_input_channel_meaning():
     assert torch.all(x[0, 2] == 1) and torch.all(x[1, 2] == 0)
     assert x[1, 0, 0, 0] == 1 and x[1, 1, 18, 18] == 1          # colours swap with the side to move
     assert torch.equal(R.legal_from_input(x), boards.view(2, -1).eq(0))   # vector_env.py:95-96
+
+
+def test_oracle_reproduces_committed_golden_vectors():
+    import numpy as np
+    from pathlib import Path
+
+    g = np.load(Path(__file__).resolve().parent / "golden" / "default_arch_golden.npz")
+    x, legal = gen_boards(6, 200, 2025)
+    assert np.array_equal(g["x"], x.numpy()) and np.array_equal(g["legal"], legal.numpy())
+    for init in ("reference", "torch_default"):
+        logits, value = R.forward(R.init_state(1234, init), x)
+        assert np.allclose(g[f"{init}_logits"], logits.numpy(), rtol=1e-5, atol=1e-7)
+        assert np.allclose(g[f"{init}_value"], value.numpy(), rtol=1e-5, atol=1e-7)
+        a, lp = R.sample_inverse_cdf(logits, legal, torch.from_numpy(g["u"]), 1.0)
+        assert np.array_equal(g[f"{init}_actions"], a.numpy())
