@@ -232,3 +232,13 @@ def test_symmetry_helpers_on_host():
             ob, oa = c6.transform_boards(b, k, flip), int(c6.transform_actions(a, n, k, flip))
             assert int(ob[0, oa // n, oa % n]) == 1
             assert torch.equal(c6.inverse_transform_actions(torch.tensor([oa]), n, k, flip), a)
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    # there is no fallback path: without the built shared object every entry raises
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "_SO", tmp_path / "libconnect6_amd.so")
+    with pytest.raises(c6.C6Error, match="no fallback"):
+        _lib.load()
+    with pytest.raises(c6.C6Error):
+        _lib.packed_bytes(_lib.PREC_BF16)
