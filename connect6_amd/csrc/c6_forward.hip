@@ -170,6 +170,7 @@ template <class P> struct L1Pipe {
   static_assert(U % D == 0 && ITERS * ROWS_BODY == kL1RowsHalf, "first-layer pipeline shape");
 };
 
+// fragments (k-step s, cout tile t) of a layer with NT cout tiles sit at index s*NT + t
 template <int D, int NT>
 __device__ __forceinline__ void preload_ring(v4i (&ring)[D][NT], const v4i *__restrict__ wl) {
 #pragma unroll
@@ -183,21 +184,8 @@ __device__ __forceinline__ const v4i *layer_weights(const unsigned char *packed,
   return reinterpret_cast<const v4i *>(packed + (size_t)Geo<P>::frag_offset(L) * 1024) + lane;
 }
 
-// ------------------------------------------------------------------------
-// K-loops.  Each layer runs as two passes over K: pass A accumulates pixel
-// tiles 0 and 1, pass B pixel tile 2.  While pass B's MFMAs run, the same wave
-// applies SiLU to pass A's finished accumulators ("side work"), so two thirds
-// of the epilogue's VALU work hides under matrix-core time.  Pass A's weight
-// prefetch wraps around so that pass B starts with a full ring.
-// ------------------------------------------------------------------------
-// Two-pass K-loops (pixel tiles {0,1} then {2} with the epilogue of the first pass riding
-// along) were measured slower than one pass: the second pass re-streams every weight
-// fragment for a third of the MFMA work and becomes L1-bound.  Kept switchable.
-constexpr bool kTwoPass = false;
-
 // Issue order inside one k-step: memory instructions are dealt out one at a time between
-// MFMAs.  Issued back to back, three ds_read_b128 or global_load_dwordx4 hold the wave's
-// issue port longer than one MFMA executes and the matrix pipe runs dry.
+// MFMAs instead of in a burst.
 template <int N_MFMA, int N_DSREAD, int N_VMEM> __device__ __forceinline__ void interleave_step() {
 #pragma unroll
   for (int i = 0; i < N_MFMA; ++i) {
@@ -210,55 +198,53 @@ template <int N_MFMA, int N_DSREAD, int N_VMEM> __device__ __forceinline__ void 
   }
 }
 
-struct NoSide {
-  __device__ __forceinline__ void operator()(int) const {}
-};
-
+// ------------------------------------------------------------------------
 // first layer: 23x23 on 3 planes, K = (ky, plane, kx24) split over lane halves
-template <class P, int J0, int NJ, bool WRAP, bool UNROLL, class Side>
+// ------------------------------------------------------------------------
+template <class P>
 __device__ __forceinline__ void conv1_pass(const unsigned char *smem, const v4i *__restrict__ wl,
                                            v4i (&ring)[L1Pipe<P>::D][1], const int (&l1base)[3],
-                                           f32x16 (&acc)[1][3], Side side) {
+                                           f32x16 (&acc)[1][3]) {
   using G = Geo<P>;
   using PP = L1Pipe<P>;
   constexpr int CPR = PP::CPR, U = PP::U, D = PP::D, ITERS = PP::ITERS;
   constexpr int ROWB = kL1RowPitch * G::EB;
 
-  v4i bcur[NJ];
+  v4i bcur[3];
 #pragma unroll
-  for (int j = 0; j < NJ; ++j) bcur[j] = *reinterpret_cast<const v4i *>(smem + l1base[J0 + j]);
-#pragma unroll(UNROLL ? ITERS : 1)
+  for (int j = 0; j < 3; ++j) bcur[j] = *reinterpret_cast<const v4i *>(smem + l1base[j]);
+#pragma unroll 1
   for (int it = 0; it < ITERS; ++it) {
     const int adv = it * PP::ROWS_BODY * ROWB;
-    const v4i *wlo = wl + (size_t)(it * U + D) * 64;
-    const v4i *whi = (WRAP && it == ITERS - 1) ? wl - (size_t)(U - D) * 64 : wlo;
+    const v4i *wn = wl + (size_t)(it * U + D) * 64;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       // operand fragments of the NEXT k-step are fetched while this step's MFMAs run; after
       // the last step this reads the zero row / the next copy, which is harmless
       const int un = u + 1;
       const int offn = (un / CPR) * ROWB + (un % CPR) * 16;
-      v4i bnext[NJ];
+      v4i bnext[3];
 #pragma unroll
-      for (int j = 0; j < NJ; ++j)
-        bnext[j] = *reinterpret_cast<const v4i *>(smem + l1base[J0 + j] + adv + offn);
+      for (int j = 0; j < 3; ++j)
+        bnext[j] = *reinterpret_cast<const v4i *>(smem + l1base[j] + adv + offn);
 #pragma unroll
-      for (int j = 0; j < NJ; ++j) mma<P>(ring[u % D][0], bcur[j], acc[0][J0 + j]);
-      ring[u % D][0] = (u < U - D ? wlo : whi)[u * 64];  // k-step it*U + u + D (wrapped or over-read)
-      side(it * U + u);
-      interleave_step<NJ * (P::EB == 4 ? 4 : 1), NJ, 1>();
+      for (int j = 0; j < 3; ++j) mma<P>(ring[u % D][0], bcur[j], acc[0][j]);
+      ring[u % D][0] = wn[u * 64];  // k-step it*U + u + D (the tail over-reads the next layer)
+      interleave_step<3 * (P::EB == 4 ? 4 : 1), 3, 1>();
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int j = 0; j < NJ; ++j) bcur[j] = bnext[j];
+      for (int j = 0; j < 3; ++j) bcur[j] = bnext[j];
     }
   }
 }
 
+// ------------------------------------------------------------------------
 // 3x3 layers: K = (tap, cin), cin fastest; taps are constant position offsets
-template <class P, int CIN, int COUT, int J0, int NJ, bool WRAP, bool UNROLL, class Side>
+// ------------------------------------------------------------------------
+template <class P, int CIN, int COUT>
 __device__ __forceinline__ void conv3_pass(const unsigned char *smem, const v4i *__restrict__ wl,
-                                           v4i (&ring)[kRing][COUT / 32], const int (&ci)[3],
-                                           int h, f32x16 (&acc)[COUT / 32][3], Side side) {
+                                           v4i (&ring)[kRing][COUT / 32], const int (&ci)[3], int h,
+                                           f32x16 (&acc)[COUT / 32][3]) {
   using G = Geo<P>;
   constexpr int NT = COUT / 32;
   constexpr int KC = CIN / G::KSTEP;
@@ -267,13 +253,13 @@ __device__ __forceinline__ void conv3_pass(const unsigned char *smem, const v4i 
   static_assert(U % D == 0, "ring depth must divide the k-steps of a kernel row");
 
   // LDS address of logical record offset `o` at tap (j, kx): pb + (x ^ o), x = lane-half ^ swizzle
-  int pb[NJ][3], xo[NJ][3];
+  int pb[3][3], xo[3][3];
   auto set_row = [&](int ky) {
 #pragma unroll
-    for (int j = 0; j < NJ; ++j)
+    for (int j = 0; j < 3; ++j)
 #pragma unroll
       for (int kx = 0; kx < 3; ++kx) {
-        const int pos = ci[J0 + j] + (ky - 1) * kPitch + (kx - 1);
+        const int pos = ci[j] + (ky - 1) * kPitch + (kx - 1);
         pb[j][kx] = pos * G::PIXB;
         xo[j][kx] = (h << 4) ^ swz_of<P>(pos);
       }
@@ -286,17 +272,16 @@ __device__ __forceinline__ void conv3_pass(const unsigned char *smem, const v4i 
     }
   };
   set_row(0);
-  v4i bcur[NJ], lcur[NJ];
+  v4i bcur[3], lcur[3];
 #pragma unroll
-  for (int j = 0; j < NJ; ++j) {
+  for (int j = 0; j < 3; ++j) {
     bcur[j] = frag_at(j, 0, 0);
     if constexpr (P::SPLIT) lcur[j] = frag_at(j, 0, G::PLANE);
   }
 
-#pragma unroll(UNROLL ? 3 : 1)
+#pragma unroll 1
   for (int ky = 0; ky < 3; ++ky) {
-    const v4i *wlo = wl + (size_t)(ky * U + D) * NT * 64;
-    const v4i *whi = (WRAP && ky == 2) ? wl - (size_t)(U - D) * NT * 64 : wlo;
+    const v4i *wn = wl + (size_t)(ky * U + D) * NT * 64;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       // fetch the activation fragments of the next k-step while this step's MFMAs run
@@ -304,39 +289,29 @@ __device__ __forceinline__ void conv3_pass(const unsigned char *smem, const v4i 
       if (u + 1 == U) set_row(ky == 2 ? 0 : ky + 1);
       const int kxn = (u + 1 < U) ? (u + 1) / KC : 0;
       const int on = (u + 1 < U) ? ((u + 1) % KC) * 32 : 0;
-      v4i bnext[NJ], lnext[NJ];
+      v4i bnext[3], lnext[3];
 #pragma unroll
-      for (int j = 0; j < NJ; ++j) {
+      for (int j = 0; j < 3; ++j) {
         bnext[j] = frag_at(j, kxn, on);
         if constexpr (P::SPLIT) lnext[j] = frag_at(j, kxn, on + G::PLANE);
       }
 #pragma unroll
       for (int t = 0; t < NT; ++t)
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) mma<P>(ring[u % D][t], bcur[j], acc[t][J0 + j]);
+        for (int j = 0; j < 3; ++j) mma<P>(ring[u % D][t], bcur[j], acc[t][j]);
       if constexpr (P::SPLIT) {
 #pragma unroll
         for (int t = 0; t < NT; ++t)
 #pragma unroll
-          for (int j = 0; j < NJ; ++j) mma<P>(ring[u % D][t], lcur[j], acc[t][J0 + j]);
+          for (int j = 0; j < 3; ++j) mma<P>(ring[u % D][t], lcur[j], acc[t][j]);
       }
-      // weights of k-step u+D (wrapped to the layer start, or over-reading into the next layer)
-#if defined(C6_EXP_FEWLOADS)   // tuning experiment only: a third of the weight traffic (wrong results)
-      ring[u % D][0] = (u < U - D ? wlo : whi)[(u * NT) * 64];
+      // weights of k-step u+D (the tail over-reads into the next layer)
 #pragma unroll
-      for (int t = 1; t < NT; ++t) ring[u % D][t] = ring[u % D][0];
-#elif defined(C6_EXP_SAMEADDR)  // tuning experiment only: every load hits the same lines (wrong results)
-#pragma unroll
-      for (int t = 0; t < NT; ++t) ring[u % D][t] = wl[t * 64 + (u & 1) * 4096];
-#else
-#pragma unroll
-      for (int t = 0; t < NT; ++t) ring[u % D][t] = (u < U - D ? wlo : whi)[(u * NT + t) * 64];
-#endif
-      side(ky * U + u);
-      interleave_step<NT * NJ * (P::SPLIT ? 2 : 1) * (P::EB == 4 ? 4 : 1), NJ * (P::SPLIT ? 2 : 1), NT>();
+      for (int t = 0; t < NT; ++t) ring[u % D][t] = wn[(u * NT + t) * 64];
+      interleave_step<NT * 3 * (P::SPLIT ? 2 : 1) * (P::EB == 4 ? 4 : 1), 3 * (P::SPLIT ? 2 : 1), NT>();
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int j = 0; j < NJ; ++j) {
+      for (int j = 0; j < 3; ++j) {
         bcur[j] = bnext[j];
         if constexpr (P::SPLIT) lcur[j] = lnext[j];
       }
@@ -405,8 +380,8 @@ __device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
 #pragma unroll
         for (int j = 0; j < 3; ++j) {
           const v8i b = __builtin_shufflevector(bcur[j][0], bcur[j][1], 0, 1, 2, 3, 4, 5, 6, 7);
-          acc[t][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[t][j], 0, 0, 0, scale_w, 0,
-                                                                      scale_x);
+          acc[t][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[t][j], 0, 0, 0,
+                                                                           scale_w, 0, scale_x);
         }
       }
       // weights of chunk c0 + d + D (the tail over-reads the next layer's copy or the zero padding)
@@ -414,15 +389,7 @@ __device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
       for (int t = 0; t < NT; ++t)
 #pragma unroll
         for (int pc = 0; pc < 2; ++pc) ring[d][t][pc] = wn[((d * NT + t) * 2 + pc) * 64];
-#pragma unroll
-      for (int i = 0; i < NT * 3; ++i) {  // one memory instruction between consecutive MFMAs
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        if (i < 6) {
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        } else if (i < 6 + NT * 2) {
-          __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-        }
-      }
+      interleave_step<NT * 3, 2 * 3, 2 * NT>();
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int j = 0; j < 3; ++j) {
@@ -442,12 +409,13 @@ __device__ __forceinline__ Packed4<P> silu_quad(const f32x16 (&acc)[NT][3], int 
   return pack4<P>(v);
 }
 
-// Write one pixel tile's packed activations.  Lanes beyond pixel 360 shadow pixel 360 (same
-// inputs, same results, same address), so every lane stores unconditionally.  The lane's
-// addresses are recomputed here every time: hoisted out of the board loop they would occupy
-// ~100 registers for the whole kernel and end up in scratch memory.
-template <class P, int NT, class Get>
-__device__ __forceinline__ void store_tile(unsigned char *smem, int pos_in, int h, Get get) {
+// SiLU + store of one pixel tile's accumulators (all cout tiles).  Lanes beyond pixel
+// 360 shadow pixel 360 (same inputs, same results, same address), so every lane stores
+// unconditionally.  The lane's addresses are recomputed here every time: hoisted out of the
+// board loop they would occupy ~100 registers for the whole kernel and end up in scratch.
+template <class P, int NT>
+__device__ __forceinline__ void store_tile(unsigned char *smem, int pos_in, int h,
+                                           const f32x16 (&acc)[NT][3], int j) {
   using G = Geo<P>;
   int pos = pos_in;
   asm volatile("" : "+v"(pos));
@@ -456,7 +424,8 @@ __device__ __forceinline__ void store_tile(unsigned char *smem, int pos_in, int 
 #pragma unroll
   for (int t = 0; t < NT; ++t)
 #pragma unroll
-    for (int q = 0; q < 4; ++q) put4<P>(smem, pbase, sw, (32 * t + 8 * q + 4 * h) * G::EB, get(t, q));
+    for (int q = 0; q < 4; ++q)
+      put4<P>(smem, pbase, sw, (32 * t + 8 * q + 4 * h) * G::EB, silu_quad<P, NT>(acc, t, j, q));
 }
 
 // accumulators start at the layer's bias: lane (h) register i holds channel 32t + 8(i/4) + 4h + i%4
@@ -476,80 +445,46 @@ __device__ __forceinline__ void init_acc(f32x16 (&acc)[N][3], const float *__res
     }
 }
 
-// barrier; pass A's packed activations and pass B's (SiLU here) go to the tile; barrier
+// barrier; every wave writes its share of the layer's output over the layer's input; barrier
 template <class P, int NT, class Pre>
 __device__ __forceinline__ void finish_layer(unsigned char *smem, const int (&ci)[3], int h,
-                                             const f32x16 (&acc)[NT][3],
-                                             const Packed4<P> (&pk)[2][NT][4], Pre before_store) {
+                                             const f32x16 (&acc)[NT][3], Pre before_store) {
   __syncthreads();  // every wave has finished reading the layer's input
   before_store();
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    if constexpr (kTwoPass) {
-      store_tile<P, NT>(smem, ci[j], h, [&](int t, int q) { return pk[j][t][q]; });
-    } else {
-      store_tile<P, NT>(smem, ci[j], h, [&](int t, int q) { return silu_quad<P, NT>(acc, t, j, q); });
-    }
-  }
-  store_tile<P, NT>(smem, ci[2], h, [&](int t, int q) { return silu_quad<P, NT>(acc, t, 2, q); });
+  for (int j = 0; j < 3; ++j) store_tile<P, NT>(smem, ci[j], h, acc, j);
   __syncthreads();
 }
 
-// side work of pass B: SiLU + pack of pass A's accumulators, one quad per k-step
-template <class P, int NT> struct SiluSide {
-  const f32x16 (&acc)[NT][3];
-  Packed4<P> (&pk)[2][NT][4];
-  __device__ __forceinline__ void operator()(int step) const {
-    if (step < 8 * NT) {
-      const int j = step / (4 * NT), t = (step / 4) % NT, q = step % 4;
-      pk[j][t][q] = silu_quad<P, NT>(acc, t, j, q);
-    }
-  }
-};
-
 // one 3x3 layer that is not the last
-template <class P, int L, int NTN>
-__device__ __forceinline__ void mid_layer(unsigned char *smem, const unsigned char *packed,
-                                          const float *tail,
-                                          v4i (&ring)[kRing][kCoutArr[L] / 32],
-                                          v4i (&next)[kRing][NTN], const int (&ci)[3], int h,
-                                          int lane, bool trace_on = false) {
+template <class P, int L>
+__device__ __forceinline__ void mid_layer(
+    unsigned char *smem, const unsigned char *packed, const float *tail,
+    v4i (&ring)[kRing][kCoutArr[L] / 32], v4i (&next)[kRing][kCoutArr[L + 1] / 32],
+    const int (&ci)[3], int h, int lane, int wave, bool trace_on) {
   constexpr int CIN = kCinArr[L], COUT = kCoutArr[L], NT = COUT / 32;
-  static_assert(NTN == kCoutArr[L + 1] / 32, "ring shape of the following layer");
   f32x16 acc[NT][3];
-  Packed4<P> pk[2][NT][4];
   init_acc(acc, tail + bias_offset(L), h);
-  const v4i *wl = layer_weights<P, L>(packed, lane);
-  if constexpr (kTwoPass) {
-    conv3_pass<P, CIN, COUT, 0, 2, true, false>(smem, wl, ring, ci, h, acc, NoSide{});
-    conv3_pass<P, CIN, COUT, 2, 1, false, true>(smem, wl, ring, ci, h, acc, SiluSide<P, NT>{acc, pk});
-  } else {
-    conv3_pass<P, CIN, COUT, 0, 3, false, false>(smem, wl, ring, ci, h, acc, NoSide{});
-  }
+  conv3_pass<P, CIN, COUT>(smem, layer_weights<P, L>(packed, lane), ring, ci, h, acc);
   if constexpr (P::LO8) conv3_lo_pass<P, L>(smem, packed, tail, ci, h, lane, acc);
-  preload_ring(next, layer_weights<P, L + 1>(packed, lane));
-#ifdef C6_TRACE
-  {
-    const int wave = threadIdx.x >> 6;
-    C6_MARK(4 + 2 * L);
-  }
-#endif
-  finish_layer<P, NT>(smem, ci, h, acc, pk, [] {});
-#ifdef C6_TRACE
-  {
-    const int wave = threadIdx.x >> 6;
-    C6_MARK(5 + 2 * L);
-  }
-#endif
+  preload_ring<kRing, kCoutArr[L + 1] / 32>(next, layer_weights<P, L + 1>(packed, lane));
+  C6_MARK(4 + 2 * L);
+  finish_layer<P, NT>(smem, ci, h, acc, [] {});
+  C6_MARK(5 + 2 * L);
+  (void)wave;
+  (void)trace_on;
 }
 
 // ------------------------------------------------------------------------
-// the fused kernel
+// the fused kernel: a persistent loop over boards; one wave per SIMD, each wave owning all
+// output channels of its 96 pixels
 // ------------------------------------------------------------------------
 template <class P>
-__global__ __launch_bounds__(kThreads) void fused_forward_kernel(const FwdParams prm) {
+__global__ __launch_bounds__(256) void fused_forward_kernel(const FwdParams prm) {
   using G = Geo<P>;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  constexpr int THREADS = 256, NWAVES = THREADS / 64;
+  constexpr int ROUNDS = (kPix + THREADS - 1) / THREADS;  // pixels per thread when staging
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -557,7 +492,7 @@ __global__ __launch_bounds__(kThreads) void fused_forward_kernel(const FwdParams
   const int h = lane >> 5;
   const int n = lane & 31;
 
-  // per-lane pixel geometry of the three 32-pixel tiles this wave owns
+  // per-lane pixel geometry of the three 32-pixel tiles of this quarter
   int ci[3], l1base[3], pix[3];
   bool valid[3];
 #pragma unroll
@@ -580,9 +515,9 @@ __global__ __launch_bounds__(kThreads) void fused_forward_kernel(const FwdParams
   auto packed_of = [&](long long b) {
     return prm.packed + (size_t)((unsigned)b / per_group) * prm.packed_stride;
   };
-  // input of one board: each thread owns pixels tid and tid+256 (three planes + occupancy)
-  float xin[2][3];
-  unsigned char occin[2];
+  // input of one board: each thread owns pixels tid, tid + THREADS, ... (three planes + occupancy)
+  float xin[ROUNDS][3];
+  unsigned char occin[ROUNDS];
   auto fetch_board = [&](long long b) {
     if (prm.x_dtype == C6_DT_BOARD_I8) {
       // environment state in, network planes out (connect6/vector_env.py:196-218 of the
@@ -593,8 +528,8 @@ __global__ __launch_bounds__(kThreads) void fused_forward_kernel(const FwdParams
       const int me = prm.player[src];
       const float last = prm.stones_left[src] == 1 ? 1.0f : 0.0f;
 #pragma unroll
-      for (int r = 0; r < 2; ++r) {
-        const int p = tid + r * kThreads;
+      for (int r = 0; r < ROUNDS; ++r) {
+        const int p = tid + r * THREADS;
         if (p < kPix) {
           const int stone = board[prm.view ? d4_from_view(p, prm.view) : p];
           xin[r][0] = stone == me ? 1.0f : 0.0f;
@@ -606,8 +541,8 @@ __global__ __launch_bounds__(kThreads) void fused_forward_kernel(const FwdParams
       return;
     }
 #pragma unroll
-    for (int r = 0; r < 2; ++r) {
-      const int p = tid + r * kThreads;
+    for (int r = 0; r < ROUNDS; ++r) {
+      const int p = tid + r * THREADS;
       if (p < kPix) {
 #pragma unroll
         for (int ch = 0; ch < 3; ++ch)
@@ -620,7 +555,7 @@ __global__ __launch_bounds__(kThreads) void fused_forward_kernel(const FwdParams
   long long b = blockIdx.x;
   if (b >= prm.total_boards) return;
   v4i r1[L1Pipe<P>::D][1];
-  preload_ring(r1, layer_weights<P, 0>(packed_of(b), lane));
+  preload_ring<L1Pipe<P>::D, 1>(r1, layer_weights<P, 0>(packed_of(b), lane));
   fetch_board(b);
 
   for (; b < prm.total_boards; b += gridDim.x) {
@@ -633,20 +568,19 @@ __global__ __launch_bounds__(kThreads) void fused_forward_kernel(const FwdParams
     const bool trace_on = (b == blockIdx.x + 2LL * gridDim.x);  // third board of this workgroup
 #else
     const bool trace_on = false;
-    (void)trace_on;
 #endif
     __syncthreads();  // previous board fully written out; LDS is free
     C6_MARK(0);
     // ---- stage the input: zero the shifted copies, then scatter the board ----
     {
       const v4i z = {0, 0, 0, 0};
-      for (int i = tidv * 16; i < G::COPIES_BYTES; i += kThreads * 16)
+      for (int i = tidv * 16; i < G::COPIES_BYTES; i += THREADS * 16)
         *reinterpret_cast<v4i *>(smem + i) = z;
     }
     __syncthreads();
 #pragma unroll
-    for (int r = 0; r < 2; ++r) {
-      const int p = tidv + r * kThreads;
+    for (int r = 0; r < ROUNDS; ++r) {
+      const int p = tidv + r * THREADS;
       if (p < kPix) {
         const int row = p / kBoard, c = p - row * kBoard;
         unsigned char o = occin[r];
@@ -677,20 +611,13 @@ __global__ __launch_bounds__(kThreads) void fused_forward_kernel(const FwdParams
     // ---- layer 1 ----
     {
       f32x16 acc[1][3];
-      Packed4<P> pk[2][1][4];
       init_acc(acc, tail + bias_offset(0), h);
-      const v4i *wl = layer_weights<P, 0>(packed, lane);
-      if constexpr (kTwoPass) {
-        conv1_pass<P, 0, 2, true, false>(smem, wl, r1, l1base, acc, NoSide{});
-        conv1_pass<P, 2, 1, false, true>(smem, wl, r1, l1base, acc, SiluSide<P, 1>{acc, pk});
-      } else {
-        conv1_pass<P, 0, 3, false, false>(smem, wl, r1, l1base, acc, NoSide{});
-      }
-      preload_ring(r2, layer_weights<P, 1>(packed, lane));
+      conv1_pass<P>(smem, layer_weights<P, 0>(packed, lane), r1, l1base, acc);
+      preload_ring<kRing, 1>(r2, layer_weights<P, 1>(packed, lane));
       C6_MARK(2);
-      finish_layer<P, 1>(smem, ci, h, acc, pk, [&] {
+      finish_layer<P, 1>(smem, ci, h, acc, [&] {
         // the copies overlapped the activation tile: restore its zero padding
-        for (int i = tidv; i < 60 * (G::PIXB / 16); i += kThreads) {
+        for (int i = tidv; i < 60 * (G::PIXB / 16); i += THREADS) {
           const int k = i / (G::PIXB / 16), w16 = i - k * (G::PIXB / 16);
           // pad positions: 0..19 (top row), 400..420 (bottom row + tail), 20*R (left column)
           const int pos = k < 20 ? k : (k < 41 ? 400 + (k - 20) : (k - 40) * kPitch);
@@ -700,12 +627,12 @@ __global__ __launch_bounds__(kThreads) void fused_forward_kernel(const FwdParams
       });
     }
     C6_MARK(3);
-    mid_layer<P, 1, 2>(smem, packed, tail, r2, r3, ci, h, lane, trace_on);
-    mid_layer<P, 2, 2>(smem, packed, tail, r3, r4, ci, h, lane, trace_on);
-    mid_layer<P, 3, 2>(smem, packed, tail, r4, r5, ci, h, lane, trace_on);
-    mid_layer<P, 4, 3>(smem, packed, tail, r5, r6, ci, h, lane, trace_on);
-    mid_layer<P, 5, 3>(smem, packed, tail, r6, r7, ci, h, lane, trace_on);
-    mid_layer<P, 6, 3>(smem, packed, tail, r7, r8, ci, h, lane, trace_on);
+    mid_layer<P, 1>(smem, packed, tail, r2, r3, ci, h, lane, wave, trace_on);
+    mid_layer<P, 2>(smem, packed, tail, r3, r4, ci, h, lane, wave, trace_on);
+    mid_layer<P, 3>(smem, packed, tail, r4, r5, ci, h, lane, wave, trace_on);
+    mid_layer<P, 4>(smem, packed, tail, r5, r6, ci, h, lane, wave, trace_on);
+    mid_layer<P, 5>(smem, packed, tail, r6, r7, ci, h, lane, wave, trace_on);
+    mid_layer<P, 6>(smem, packed, tail, r7, r8, ci, h, lane, wave, trace_on);
 
     // ---- layer 8 + both 1x1 heads straight from the fp32 accumulators ----
     {
@@ -715,54 +642,44 @@ __global__ __launch_bounds__(kThreads) void fused_forward_kernel(const FwdParams
       const float *valw = polw + kHeadC;
       const float *pwl = polw + 4 * h;  // per-lane base: channel 32t + 8q + 4h + e
       asm volatile("" : "+v"(pwl));
+      conv3_pass<P, 96, 96>(smem, layer_weights<P, 7>(packed, lane), r8, ci, h, acc);
+      if constexpr (P::LO8) conv3_lo_pass<P, 7>(smem, packed, tail, ci, h, lane, acc);
+      if (bn < prm.total_boards) preload_ring<L1Pipe<P>::D, 1>(r1, layer_weights<P, 0>(packed_of(bn), lane));
+      C6_MARK(18);
       float pol[3] = {0.0f, 0.0f, 0.0f};
       float vsum = 0.0f;
-      // heads of pixel tile j, quad (t, q): policy dot and value dot of four channels
-      auto head_quad = [&](int t, int j, int q) {
-        const f32x4 pw = *reinterpret_cast<const f32x4 *>(pwl + 32 * t + 8 * q);
-        const f32x4 vw = *reinterpret_cast<const f32x4 *>(pwl + kHeadC + 32 * t + 8 * q);
-        float vs = 0.0f;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const float a = silu<P>(acc[t][j][4 * q + e]);
-          pol[j] = fmaf(a, pw[e], pol[j]);
-          vs = fmaf(a, vw[e], vs);
-        }
-        vsum += valid[j] ? vs : 0.0f;
-      };
-      const v4i *wl = layer_weights<P, 7>(packed, lane);
-      if constexpr (kTwoPass) {
-        conv3_pass<P, 96, 96, 0, 2, true, false>(smem, wl, r8, ci, h, acc, NoSide{});
-        conv3_pass<P, 96, 96, 2, 1, false, true>(smem, wl, r8, ci, h, acc, [&](int step) {
-          if (step < 24) head_quad((step / 4) % 3, step / 12, step % 4);
-        });
-      } else {
-        conv3_pass<P, 96, 96, 0, 3, false, false>(smem, wl, r8, ci, h, acc, NoSide{});
-      }
-      if constexpr (P::LO8) conv3_lo_pass<P, 7>(smem, packed, tail, ci, h, lane, acc);
-      if (bn < prm.total_boards) preload_ring(r1, layer_weights<P, 0>(packed_of(bn), lane));
-      C6_MARK(18);
-#pragma unroll
-      for (int j = 0; j < (kTwoPass ? 0 : 2); ++j)
-#pragma unroll
-        for (int t = 0; t < 3; ++t)
-#pragma unroll
-          for (int q = 0; q < 4; ++q) head_quad(t, j, q);
 #pragma unroll
       for (int t = 0; t < 3; ++t)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) head_quad(t, 2, q);
-      const float polb = valw[kHeadC], valb = valw[kHeadC + 1];
+        for (int q = 0; q < 4; ++q) {
+          const f32x4 pw = *reinterpret_cast<const f32x4 *>(pwl + 32 * t + 8 * q);
+          const f32x4 vw = *reinterpret_cast<const f32x4 *>(pwl + kHeadC + 32 * t + 8 * q);
 #pragma unroll
-      for (int j = 0; j < 3; ++j) {
-        const float tot = pol[j] + __shfl_xor(pol[j], 32, 64);
-        if (h == 0 && valid[j]) lgt[pix[j]] = tot + polb;
-      }
+          for (int j = 0; j < 3; ++j) {
+            float vs = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const float a = silu<P>(acc[t][j][4 * q + e]);
+              pol[j] = fmaf(a, pw[e], pol[j]);
+              vs = fmaf(a, vw[e], vs);
+            }
+            vsum += valid[j] ? vs : 0.0f;
+          }
+        }
+      const float polb = valw[kHeadC], valb = valw[kHeadC + 1];
+      float tot[3];
+#pragma unroll
+      for (int j = 0; j < 3; ++j) tot[j] = pol[j] + __shfl_xor(pol[j], 32, 64);
+#pragma unroll
+      for (int j = 0; j < 3; ++j)
+        if (h == 0 && valid[j]) lgt[pix[j]] = tot[j] + polb;
       vsum = wave_sum(vsum);
       if (lane == 0) red[wave] = vsum;
       __syncthreads();
       if (tid == 0 && prm.value != nullptr) {
-        const float s = (red[0] + red[1]) + (red[2] + red[3]);
+        float s = 0.0f;
+#pragma unroll
+        for (int w = 0; w < NWAVES; ++w) s += red[w];
         prm.value[b] = tanhf(s * (1.0f / kPix) + valb);
       }
       C6_MARK(19);
@@ -770,7 +687,7 @@ __global__ __launch_bounds__(kThreads) void fused_forward_kernel(const FwdParams
 
     // ---- write out: masked logits, optional sampled action ----
     if (prm.logits != nullptr) {
-      for (int p = tid; p < kPix; p += kThreads) {
+      for (int p = tid; p < kPix; p += THREADS) {
         const float v = lgt[p];
         prm.logits[(size_t)b * kPix + p] = occ[p] ? prm.fill : v;
       }
@@ -948,26 +865,25 @@ template <class P> static int launch_forward(const FwdParams &fp, hipStream_t st
   static_assert(G::LDS_BYTES <= 160 * 1024, "activation tile must fit the 160 KiB LDS of a CU");
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
-  static thread_local int configured_dev[5] = {-1, -1, -1, -1, -1};
-  static thread_local int cus[5] = {0, 0, 0, 0, 0};
-  if (e == hipSuccess && configured_dev[P::ID] != dev) {
+  static thread_local int configured_dev = -1;
+  static thread_local int cus = 0;
+  if (e == hipSuccess && configured_dev != dev) {
     e = hipFuncSetAttribute(reinterpret_cast<const void *>(&fused_forward_kernel<P>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, G::LDS_BYTES);
     int n = 0;
     if (e == hipSuccess) e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
     if (e == hipSuccess) {
-      configured_dev[P::ID] = dev;
-      cus[P::ID] = n;
+      configured_dev = dev;
+      cus = n;
     }
   }
   if (e != hipSuccess) {
     set_error("fused_forward setup failed: %s", hipGetErrorString(e));
     return C6_ELAUNCH;
   }
-  long long grid = cus[P::ID] > 0 ? cus[P::ID] : 256;
+  long long grid = cus > 0 ? cus : 256;
   if (grid > fp.total_boards) grid = fp.total_boards;
-  hipLaunchKernelGGL(fused_forward_kernel<P>, dim3((unsigned)grid), dim3(kThreads), G::LDS_BYTES,
-                     st, fp);
+  hipLaunchKernelGGL(fused_forward_kernel<P>, dim3((unsigned)grid), dim3(256), G::LDS_BYTES, st, fp);
   e = hipGetLastError();
   if (e != hipSuccess) {
     set_error("fused_forward launch failed: %s", hipGetErrorString(e));
