@@ -17,9 +17,9 @@ _SO = _LIBDIR / "libconnect6_amd.so"
 _SOURCES = ("c6_forward.hip", "c6_tail.hip", "c6_generic.hip", "c6_api.hip")
 
 # arithmetic modes (include/connect6_amd.h)
-PREC_F32, PREC_BF16, PREC_F16, PREC_BF16X2, PREC_BF16F8 = 0, 1, 2, 3, 4
+PREC_F32, PREC_BF16, PREC_F16, PREC_BF16X2, PREC_BF16F8, PREC_BF16F6 = 0, 1, 2, 3, 4, 5
 PREC_BY_NAME = {"fp32": PREC_F32, "bf16": PREC_BF16, "fp16": PREC_F16, "bf16x2": PREC_BF16X2,
-                "bf16f8": PREC_BF16F8}
+                "bf16f8": PREC_BF16F8, "bf16f6": PREC_BF16F6}
 DT_F32, DT_BF16, DT_F16 = 0, 1, 2
 MASK_NONE, MASK_INPUT, MASK_LEGAL = 0, 1, 2
 

@@ -34,7 +34,7 @@ int launch_generic(const void *x, int x_dtype, long long batch, int n, int layer
 
 static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 static int elem_bytes(int dt) { return dt == C6_DT_F32 ? 4 : ((dt == C6_DT_BF16 || dt == C6_DT_F16) ? 2 : 0); }
-static bool valid_prec(int p) { return p >= C6_PREC_F32 && p <= C6_PREC_BF16F8; }
+static bool valid_prec(int p) { return p >= C6_PREC_F32 && p <= C6_PREC_BF16F6; }
 
 }  // namespace c6
 

@@ -60,30 +60,42 @@ struct PrecF32 {
   static constexpr int EB = 4;        // bytes per element
   static constexpr int SPLIT = 0;
   static constexpr int LO8 = 0;
+  static constexpr int LO6 = 0;
 };
 struct PrecBF16 {
   static constexpr int ID = C6_PREC_BF16;
   static constexpr int EB = 2;
   static constexpr int SPLIT = 0;
   static constexpr int LO8 = 0;
+  static constexpr int LO6 = 0;
 };
 struct PrecF16 {
   static constexpr int ID = C6_PREC_F16;
   static constexpr int EB = 2;
   static constexpr int SPLIT = 0;
   static constexpr int LO8 = 0;
+  static constexpr int LO6 = 0;
 };
 struct PrecBF16X2 {
   static constexpr int ID = C6_PREC_BF16X2;
   static constexpr int EB = 2;
   static constexpr int SPLIT = 1;     // activations stored as hi plane + lo plane, both bf16
   static constexpr int LO8 = 0;
+  static constexpr int LO6 = 0;
 };
 struct PrecBF16F8 {
   static constexpr int ID = C6_PREC_BF16F8;
   static constexpr int EB = 2;
   static constexpr int SPLIT = 0;
   static constexpr int LO8 = 1;       // bf16 plane + the dropped low-order part as scaled fp8
+  static constexpr int LO6 = 0;
+};
+struct PrecBF16F6 {
+  static constexpr int ID = C6_PREC_BF16F6;
+  static constexpr int EB = 2;
+  static constexpr int SPLIT = 0;
+  static constexpr int LO8 = 1;       // same record and fragment geometry as the fp8 mode ...
+  static constexpr int LO6 = 1;       // ... with the low-order part as block-scaled fp6 (e2m3)
 };
 
 // bf16 + fp8 mode: what rounding an activation to bf16 drops (|lo| <= 2^-9 |a|) is kept as
@@ -92,7 +104,25 @@ struct PrecBF16F8 {
 // The weight copy of layer l is scaled by 2^sw[l] (sw in the packed tail, from max|w|); the
 // instruction's block scales undo both factors.
 constexpr int kLoScaleLog2 = 12;
-constexpr int kLoRing = 3;            // fp8 weight prefetch depth (64-wide K chunks)
+constexpr int kLoRing = 3;            // low-order weight prefetch ring depth (64-wide K chunks)
+
+// bf16 + fp6 mode: the same second pass with e2m3 operands (K = 64 per instruction at four
+// times the bf16 rate).  The 32 bytes that hold 32 low-order values of a position are 24 bytes
+// of packed 6-bit values, one E8M0 scale byte (the block's power-of-two scale, taken from the
+// largest of the 32 values) and padding; the instruction applies the scale per lane.  Which 32
+// channels form a block follows from which lane holds them after the MFMA (lo6_channel).
+__host__ __device__ constexpr int lo6_channel(int cin, int block, int slot) {
+  const int i = slot >> 1, odd = slot & 1;
+  int t, hh;
+  if (cin == 32) {          // one block: both lane halves of cout tile 0, gathered in one lane
+    t = 0, hh = odd;
+  } else if (block < 2) {   // block = lane half; even slots cout tile 0, odd slots cout tile 1
+    t = odd, hh = block;
+  } else {                  // 96 channels: third block = both lane halves of cout tile 2
+    t = 2, hh = odd;
+  }
+  return 32 * t + 8 * (i >> 2) + 4 * hh + (i & 3);
+}
 
 template <class P> struct Geo {
   static constexpr int EB = P::EB;

@@ -44,6 +44,9 @@ template <> __device__ __forceinline__ void mma<PrecBF16X2>(const v4i &a, const 
 template <> __device__ __forceinline__ void mma<PrecBF16F8>(const v4i &a, const v4i &b, f32x16 &c) {
   mma<PrecBF16>(a, b, c);
 }
+template <> __device__ __forceinline__ void mma<PrecBF16F6>(const v4i &a, const v4i &b, f32x16 &c) {
+  mma<PrecBF16>(a, b, c);
+}
 template <> __device__ __forceinline__ void mma<PrecF16>(const v4i &a, const v4i &b, f32x16 &c) {
   c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
                                              __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
@@ -108,7 +111,7 @@ template <class P> __device__ __forceinline__ Packed4<P> pack4(const float (&v)[
       r.lo[0] = pack2<P>(v[0] - bf16_lo(r.hi[0]), v[1] - bf16_hi(r.hi[0]));
       r.lo[1] = pack2<P>(v[2] - bf16_lo(r.hi[1]), v[3] - bf16_hi(r.hi[1]));
     }
-    if constexpr (P::LO8) {  // dropped low-order parts as four e4m3 bytes of lo * 2^kLoScaleLog2
+    if constexpr (P::LO8 && !P::LO6) {  // dropped low-order parts as four e4m3 bytes of lo * 2^kLoScaleLog2
       // v_cvt_scalef32_pk_fp8_f32 divides by its scale operand and turns overflow into NaN,
       // so the inputs are clamped to what 448 * 2^-kLoScaleLog2 can represent.
       constexpr float INV = 1.0f / (float)(1 << kLoScaleLog2), LIM = 448.0f * INV;
@@ -136,7 +139,7 @@ __device__ __forceinline__ void put4(unsigned char *smem, int pbase, int sw, int
     *reinterpret_cast<v2i *>(smem + pbase + (o ^ sw)) = r.hi;
     if constexpr (P::SPLIT)
       *reinterpret_cast<v2i *>(smem + pbase + ((o + Geo<P>::PLANE) ^ sw)) = r.lo;
-    if constexpr (P::LO8)  // one byte per channel: channel index = o / 2
+    if constexpr (P::LO8 && !P::LO6)  // one byte per channel: channel index = o / 2
       *reinterpret_cast<int *>(smem + pbase + Geo<P>::LO_OFF + (o >> 1)) = r.lo[0];
   }
 }
@@ -184,6 +187,8 @@ __device__ __forceinline__ const v4i *layer_weights(const unsigned char *packed,
   return reinterpret_cast<const v4i *>(packed + (size_t)Geo<P>::frag_offset(L) * 1024) + lane;
 }
 
+constexpr int kAhead = 2;  // k-steps between the LDS read of an activation fragment and its MFMAs
+
 // Issue order inside one k-step: memory instructions are dealt out one at a time between
 // MFMAs instead of in a burst.
 template <int N_MFMA, int N_DSREAD, int N_VMEM> __device__ __forceinline__ void interleave_step() {
@@ -210,30 +215,32 @@ __device__ __forceinline__ void conv1_pass(const unsigned char *smem, const v4i 
   constexpr int CPR = PP::CPR, U = PP::U, D = PP::D, ITERS = PP::ITERS;
   constexpr int ROWB = kL1RowPitch * G::EB;
 
-  v4i bcur[3];
+  // activation fragments are fetched kAhead k-steps before their MFMAs (an LDS read issued
+  // during one k-step of three MFMAs would not be back by the next)
+  static_assert(U % (kAhead + 1) == 0, "fragment queue must line up across loop iterations");
+  v4i bq[kAhead + 1][3];
 #pragma unroll
-  for (int j = 0; j < 3; ++j) bcur[j] = *reinterpret_cast<const v4i *>(smem + l1base[j]);
+  for (int a = 0; a < kAhead; ++a)
+#pragma unroll
+    for (int j = 0; j < 3; ++j)
+      bq[a][j] = *reinterpret_cast<const v4i *>(smem + l1base[j] + (a / CPR) * ROWB + (a % CPR) * 16);
 #pragma unroll 1
   for (int it = 0; it < ITERS; ++it) {
     const int adv = it * PP::ROWS_BODY * ROWB;
     const v4i *wn = wl + (size_t)(it * U + D) * 64;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      // operand fragments of the NEXT k-step are fetched while this step's MFMAs run; after
-      // the last step this reads the zero row / the next copy, which is harmless
-      const int un = u + 1;
+      // after the last steps this reads the zero row / the next copy, which is harmless
+      const int un = u + kAhead;
       const int offn = (un / CPR) * ROWB + (un % CPR) * 16;
-      v4i bnext[3];
 #pragma unroll
       for (int j = 0; j < 3; ++j)
-        bnext[j] = *reinterpret_cast<const v4i *>(smem + l1base[j] + adv + offn);
+        bq[un % (kAhead + 1)][j] = *reinterpret_cast<const v4i *>(smem + l1base[j] + adv + offn);
 #pragma unroll
-      for (int j = 0; j < 3; ++j) mma<P>(ring[u % D][0], bcur[j], acc[0][j]);
+      for (int j = 0; j < 3; ++j) mma<P>(ring[u % D][0], bq[u % (kAhead + 1)][j], acc[0][j]);
       ring[u % D][0] = wn[u * 64];  // k-step it*U + u + D (the tail over-reads the next layer)
       interleave_step<3 * (P::EB == 4 ? 4 : 1), 3, 1>();
       __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int j = 0; j < 3; ++j) bcur[j] = bnext[j];
     }
   }
 }
@@ -272,79 +279,107 @@ __device__ __forceinline__ void conv3_pass(const unsigned char *smem, const v4i 
     }
   };
   set_row(0);
-  v4i bcur[3], lcur[3];
+  static_assert(U % (kAhead + 1) == 0 && kAhead <= KC, "fragment queue must line up across kernel rows");
+  v4i bq[kAhead + 1][3], lq[kAhead + 1][3];
 #pragma unroll
-  for (int j = 0; j < 3; ++j) {
-    bcur[j] = frag_at(j, 0, 0);
-    if constexpr (P::SPLIT) lcur[j] = frag_at(j, 0, G::PLANE);
-  }
+  for (int a = 0; a < kAhead; ++a)
+#pragma unroll
+    for (int j = 0; j < 3; ++j) {
+      bq[a][j] = frag_at(j, 0, a * 32);
+      if constexpr (P::SPLIT) lq[a][j] = frag_at(j, 0, a * 32 + G::PLANE);
+    }
 
 #pragma unroll 1
   for (int ky = 0; ky < 3; ++ky) {
     const v4i *wn = wl + (size_t)(ky * U + D) * NT * 64;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      // fetch the activation fragments of the next k-step while this step's MFMAs run
-      // (after the last tap this wraps to kernel row 0: one harmless extra fetch)
-      if (u + 1 == U) set_row(ky == 2 ? 0 : ky + 1);
-      const int kxn = (u + 1 < U) ? (u + 1) / KC : 0;
-      const int on = (u + 1 < U) ? ((u + 1) % KC) * 32 : 0;
-      v4i bnext[3], lnext[3];
+      // fetch the activation fragments of k-step u + kAhead while this step's MFMAs run
+      // (after the last tap this wraps to kernel row 0: harmless extra fetches)
+      if (u + kAhead == U) set_row(ky == 2 ? 0 : ky + 1);
+      constexpr int QN = kAhead + 1;
+      const int un = (u + kAhead) % U;
+      const int kxn = un / KC, on = (un % KC) * 32;
 #pragma unroll
       for (int j = 0; j < 3; ++j) {
-        bnext[j] = frag_at(j, kxn, on);
-        if constexpr (P::SPLIT) lnext[j] = frag_at(j, kxn, on + G::PLANE);
+        bq[(u + kAhead) % QN][j] = frag_at(j, kxn, on);
+        if constexpr (P::SPLIT) lq[(u + kAhead) % QN][j] = frag_at(j, kxn, on + G::PLANE);
       }
 #pragma unroll
       for (int t = 0; t < NT; ++t)
 #pragma unroll
-        for (int j = 0; j < 3; ++j) mma<P>(ring[u % D][t], bcur[j], acc[t][j]);
+        for (int j = 0; j < 3; ++j) mma<P>(ring[u % D][t], bq[u % QN][j], acc[t][j]);
       if constexpr (P::SPLIT) {
 #pragma unroll
         for (int t = 0; t < NT; ++t)
 #pragma unroll
-          for (int j = 0; j < 3; ++j) mma<P>(ring[u % D][t], lcur[j], acc[t][j]);
+          for (int j = 0; j < 3; ++j) mma<P>(ring[u % D][t], lq[u % QN][j], acc[t][j]);
       }
       // weights of k-step u+D (the tail over-reads into the next layer)
 #pragma unroll
       for (int t = 0; t < NT; ++t) ring[u % D][t] = wn[(u * NT + t) * 64];
       interleave_step<NT * 3 * (P::SPLIT ? 2 : 1) * (P::EB == 4 ? 4 : 1), 3 * (P::SPLIT ? 2 : 1), NT>();
       __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int j = 0; j < 3; ++j) {
-        bcur[j] = bnext[j];
-        if constexpr (P::SPLIT) lcur[j] = lnext[j];
-      }
     }
   }
 }
 
-// Second pass of the bf16 + fp8 mode over a 3x3 layer: acc += W8 * LO8, both e4m3, K = 64
-// per MFMA.  Lane half h of chunk c contracts half-chunk g = 2c + h = (tap, 32-channel block).
-// A runtime loop over groups of D chunks (D = ring depth) keeps the compiler from hoisting
-// every fragment load of the layer to the front.
-template <class P, int L>
-__device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
-                                              const unsigned char *packed, const float *tail,
-                                              const int (&ci)[3], int h, int lane,
-                                              f32x16 (&acc)[kCoutArr[L] / 32][3]) {
-  using G = Geo<P>;
-  constexpr int NT = kCoutArr[L] / 32, PER32 = kCinArr[L] / 32;
-  constexpr int HC = G::lo_half_chunks(L), NC = G::lo_chunks(L);
-  constexpr int D = (NC % 3 == 0) ? 3 : ((NC % 2 == 0) ? 2 : NC);  // 5 -> 5, 9 -> 3, 14 -> 2
-  static_assert(D <= 5 && NC % D == 0, "fp8 weight ring shape");
-  typedef int v8i __attribute__((ext_vector_type(8)));
-  const v4i *wl = reinterpret_cast<const v4i *>(packed + (size_t)G::lo_frag_offset(L) * 1024) + lane;
-  v4i ring[D][NT][2];
+// Second pass of the bf16 + fp8 / fp6 modes over a 3x3 layer: acc += Wlo * LO, both e4m3 (or
+// both e2m3), K = 64 per MFMA.  Lane half h of chunk c contracts half-chunk g = 2c + h =
+// (tap, 32-channel block); in the fp6 mode the block's scale byte rides in dword 6 of the
+// 32 bytes the lane reads.
+//
+// Its weight ring: a lane's operand is 32 bytes (fp8) or 24 (fp6), piece 0 = 16 bytes and
+// piece 1 = 16 or 8.  (Filling the ring before the layer's main pass was measured slower: the
+// extra loads and registers cost the main pass more than the second pass gains.)
+template <class P>
+__device__ __forceinline__ void lo_load_pieces(const v4i *src, v4i &p0, v4i &p1) {
+  p0 = src[0];
+  if constexpr (P::LO6) {
+    const v2i q = *reinterpret_cast<const v2i *>(src + 64);
+    p1 = v4i{q[0], q[1], 0, 0};
+  } else {
+    p1 = src[64];
+  }
+}
+template <class P, int L> struct LoRing {
+  static constexpr int NT = kCoutArr[L] / 32;
+  static constexpr int NC = Geo<P>::lo_chunks(L);
+  static constexpr int D = P::LO8 ? (NC < kLoRing ? NC : kLoRing) : 1;  // ring depth in 64-wide chunks
+  __device__ __forceinline__ static const v4i *base(const unsigned char *packed, int lane) {
+    return reinterpret_cast<const v4i *>(packed + (size_t)Geo<P>::lo_frag_offset(L) * 1024) + lane;
+  }
+};
+template <class P, int L, int D, int NT>
+__device__ __forceinline__ void lo_preload(v4i (&f0)[D][NT], v4i (&f1)[D][NT],
+                                           const unsigned char *packed, int lane) {
+  static_assert(D == LoRing<P, L>::D && NT == LoRing<P, L>::NT, "ring shape");
+  const v4i *wl = LoRing<P, L>::base(packed, lane);
 #pragma unroll
   for (int d = 0; d < D; ++d)
 #pragma unroll
-    for (int t = 0; t < NT; ++t)
-#pragma unroll
-      for (int pc = 0; pc < 2; ++pc) ring[d][t][pc] = wl[((d * NT + t) * 2 + pc) * 64];
+    for (int t = 0; t < NT; ++t) lo_load_pieces<P>(wl + (d * NT + t) * 2 * 64, f0[d][t], f1[d][t]);
+  __builtin_amdgcn_sched_barrier(0);  // issue here: do not sink the loads to their first use
+}
+
+// A runtime loop over groups of D chunks (D = ring depth) keeps the compiler from hoisting
+// every fragment load of the layer to the front.
+template <class P, int L, int D, int NT>
+__device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
+                                              const unsigned char *packed, const float *tail,
+                                              v4i (&ring0)[D][NT], v4i (&ring1)[D][NT],
+                                              const int (&ci)[3], int h, int lane,
+                                              f32x16 (&acc)[NT][3]) {
+  using G = Geo<P>;
+  static_assert(D == LoRing<P, L>::D && NT == kCoutArr[L] / 32, "ring shape");
+  constexpr int PER32 = kCinArr[L] / 32;
+  constexpr int HC = G::lo_half_chunks(L), NC = G::lo_chunks(L);
+  typedef int v8i __attribute__((ext_vector_type(8)));
+  const v4i *wl = LoRing<P, L>::base(packed, lane);
   const int sw = reinterpret_cast<const int *>(tail)[G::TAIL_SW + L];
   const int scale_w = 127 - sw;            // E8M0 exponent undoing the weight copy's 2^sw
-  const int scale_x = 127 - kLoScaleLog2;  // ... and the activations' 2^kLoScaleLog2
+  const int scale_x = 127 - kLoScaleLog2;  // ... and the activations' 2^kLoScaleLog2 (fp8 mode)
+  (void)scale_x;
 
   int pbase[3];
 #pragma unroll
@@ -362,40 +397,51 @@ __device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
 #pragma unroll
     for (int j = 0; j < 3; ++j) {
       b[j][0] = *reinterpret_cast<const v4i *>(smem + pbase[j] + off);
-      b[j][1] = *reinterpret_cast<const v4i *>(smem + pbase[j] + off + 16);
+      if constexpr (P::LO6) {
+        // 12 bytes: the last two data dwords and the scale (a 16-byte read would leave a dead
+        // register that the compiler reuses at once, waiting for the read to land first)
+        typedef int v3i __attribute__((ext_vector_type(3)));
+        const v3i q = *reinterpret_cast<const v3i *>(smem + pbase[j] + off + 16);
+        b[j][1] = v4i{q[0], q[1], q[2], 0};
+      } else {
+        b[j][1] = *reinterpret_cast<const v4i *>(smem + pbase[j] + off + 16);
+      }
     }
   };
-  v4i bcur[3][2];
-  fetch(0, bcur);
+  // activation blocks are fetched kAhead chunks ahead, like the main pass's fragments
+  static_assert(D % (kAhead + 1) == 0 && NC > kAhead, "low-order ring and fragment queue shapes");
+  v4i bq[kAhead + 1][3][2];
+#pragma unroll
+  for (int a = 0; a < kAhead; ++a) fetch(a, bq[a]);
 #pragma unroll 1
   for (int c0 = 0; c0 < NC; c0 += D) {
     const v4i *wn = wl + (size_t)(c0 + D) * NT * 2 * 64;
 #pragma unroll
     for (int d = 0; d < D; ++d) {
-      v4i bnext[3][2];
-      fetch(c0 + d + 1 < NC ? c0 + d + 1 : NC - 1, bnext);  // (after the last chunk: a harmless re-read)
+      if (NC % D != 0 && d >= NC % D && c0 + d >= NC) continue;  // the last group may be short
+      v4i(&bcur)[3][2] = bq[d % (kAhead + 1)];
+      // (after the last chunks: harmless re-reads)
+      fetch(c0 + d + kAhead < NC ? c0 + d + kAhead : NC - 1, bq[(d + kAhead) % (kAhead + 1)]);
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
-        const v8i a = __builtin_shufflevector(ring[d][t][0], ring[d][t][1], 0, 1, 2, 3, 4, 5, 6, 7);
+        const v8i a = __builtin_shufflevector(ring0[d][t], ring1[d][t], 0, 1, 2, 3, 4, 5, 6, 7);
 #pragma unroll
         for (int j = 0; j < 3; ++j) {
           const v8i b = __builtin_shufflevector(bcur[j][0], bcur[j][1], 0, 1, 2, 3, 4, 5, 6, 7);
-          acc[t][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[t][j], 0, 0, 0,
-                                                                           scale_w, 0, scale_x);
+          if constexpr (P::LO6) {
+            acc[t][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[t][j], 2, 2, 0,
+                                                                             scale_w, 0, b[6]);
+          } else {
+            acc[t][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[t][j], 0, 0, 0,
+                                                                             scale_w, 0, scale_x);
+          }
         }
       }
       // weights of chunk c0 + d + D (the tail over-reads the next layer's copy or the zero padding)
 #pragma unroll
-      for (int t = 0; t < NT; ++t)
-#pragma unroll
-        for (int pc = 0; pc < 2; ++pc) ring[d][t][pc] = wn[((d * NT + t) * 2 + pc) * 64];
+      for (int t = 0; t < NT; ++t) lo_load_pieces<P>(wn + (d * NT + t) * 2 * 64, ring0[d][t], ring1[d][t]);
       interleave_step<NT * 3, 2 * 3, 2 * NT>();
       __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int j = 0; j < 3; ++j) {
-        bcur[j][0] = bnext[j][0];
-        bcur[j][1] = bnext[j][1];
-      }
     }
   }
 }
@@ -428,6 +474,77 @@ __device__ __forceinline__ void store_tile(unsigned char *smem, int pos_in, int 
       put4<P>(smem, pbase, sw, (32 * t + 8 * q + 4 * h) * G::EB, silu_quad<P, NT>(acc, t, j, q));
 }
 
+// fp6 mode: 32 low-order values of one position -> 24 bytes of e2m3 + the block's E8M0 scale.
+// The scale is 2^(E-2) for a largest magnitude in [2^E, 2^(E+1)), so values land in (-8, 8)
+// and the conversion saturates the few above 7.5.  even[i] goes to K slot 2i, odd[i] to 2i+1.
+typedef float f32x16v __attribute__((ext_vector_type(16)));
+typedef unsigned u32x6 __attribute__((ext_vector_type(6)));
+__device__ __forceinline__ u32x6 to_fp6_block(const f32x16v &even, const f32x16v &odd, float scale) {
+  u32x6 r = __builtin_amdgcn_cvt_scalef32_2xpk16_fp6_f32(even, odd, scale);
+  // the instruction must not write where it still reads: keep every source live past it
+  asm volatile("" : "+v"(r) : "v"(even), "v"(odd), "v"(scale));
+  return r;
+}
+__device__ __forceinline__ void lo6_block(unsigned char *dst, const float (&even)[16],
+                                          const float (&odd)[16], bool store) {
+  float m = 0.0f;
+  f32x16v a, b;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    a[i] = even[i];
+    b[i] = odd[i];
+    m = fmaxf(m, fmaxf(fabsf(even[i]), fabsf(odd[i])));
+  }
+  int sc = (__builtin_bit_cast(int, m) >> 23) - 2;  // biased exponent of the block scale
+  sc = sc < 1 ? 1 : sc;
+  const u32x6 r = to_fp6_block(a, b, __builtin_bit_cast(float, sc << 23));
+  if (store) {
+    *reinterpret_cast<v4i *>(dst) = v4i{(int)r[0], (int)r[1], (int)r[2], (int)r[3]};
+    *reinterpret_cast<v4i *>(dst + 16) = v4i{(int)r[4], (int)r[5], sc, 0};
+  }
+}
+
+// SiLU + store of one pixel tile in the fp6 mode: bf16 plane as in store_tile, then the
+// low-order blocks.  Cout tiles 0 and 1 pair up inside a lane (block = lane half); an odd
+// last tile gathers both lane halves in the lower lane (block 0 of 1, or 2 of 3).
+template <class P, int NT>
+__device__ __forceinline__ void store_tile_lo6(unsigned char *smem, int pos_in, int h,
+                                               const f32x16 (&acc)[NT][3], int j) {
+  using G = Geo<P>;
+  int pos = pos_in;
+  asm volatile("" : "+v"(pos));
+  unsigned char *rec = smem + pos * G::PIXB;
+  float lo[NT][16];
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      float v[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = silu<P>(acc[t][j][4 * q + e]);
+      const v2i hi = {pack2<P>(v[0], v[1]), pack2<P>(v[2], v[3])};
+      *reinterpret_cast<v2i *>(rec + (32 * t + 8 * q + 4 * h) * 2) = hi;
+      lo[t][4 * q + 0] = v[0] - bf16_lo(hi[0]);
+      lo[t][4 * q + 1] = v[1] - bf16_hi(hi[0]);
+      lo[t][4 * q + 2] = v[2] - bf16_lo(hi[1]);
+      lo[t][4 * q + 3] = v[3] - bf16_hi(hi[1]);
+    }
+  if constexpr (NT >= 2) lo6_block(rec + G::LO_OFF + 32 * h, lo[0], lo[1], true);
+  if constexpr (NT % 2 == 1) {
+    float own[16], other[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      // lower lanes: r[0] = own value, r[1] = the value lane + 32 holds (same pixel, channels + 4)
+      const unsigned mine = __builtin_bit_cast(unsigned, lo[NT - 1][i]);
+      const auto r = __builtin_amdgcn_permlane32_swap(mine, mine, false, false);
+      const unsigned r0 = r[0], r1 = r[1];  // (bit_cast straight from a vector element reads element 0)
+      own[i] = __builtin_bit_cast(float, r0);
+      other[i] = __builtin_bit_cast(float, r1);
+    }
+    lo6_block(rec + G::LO_OFF + 32 * (NT - 1), own, other, h == 0);
+  }
+}
+
 // accumulators start at the layer's bias: lane (h) register i holds channel 32t + 8(i/4) + 4h + i%4
 template <int N>
 __device__ __forceinline__ void init_acc(f32x16 (&acc)[N][3], const float *__restrict__ bias, int h) {
@@ -452,7 +569,13 @@ __device__ __forceinline__ void finish_layer(unsigned char *smem, const int (&ci
   __syncthreads();  // every wave has finished reading the layer's input
   before_store();
 #pragma unroll
-  for (int j = 0; j < 3; ++j) store_tile<P, NT>(smem, ci[j], h, acc, j);
+  for (int j = 0; j < 3; ++j) {
+    if constexpr (P::LO6) {
+      store_tile_lo6<P, NT>(smem, ci[j], h, acc, j);
+    } else {
+      store_tile<P, NT>(smem, ci[j], h, acc, j);
+    }
+  }
   __syncthreads();
 }
 
@@ -465,8 +588,11 @@ __device__ __forceinline__ void mid_layer(
   constexpr int CIN = kCinArr[L], COUT = kCoutArr[L], NT = COUT / 32;
   f32x16 acc[NT][3];
   init_acc(acc, tail + bias_offset(L), h);
+  v4i lor0[LoRing<P, L>::D][LoRing<P, L>::NT], lor1[LoRing<P, L>::D][LoRing<P, L>::NT];
   conv3_pass<P, CIN, COUT>(smem, layer_weights<P, L>(packed, lane), ring, ci, h, acc);
-  if constexpr (P::LO8) conv3_lo_pass<P, L>(smem, packed, tail, ci, h, lane, acc);
+  C6_MARK(30 + L);
+  if constexpr (P::LO8) lo_preload<P, L>(lor0, lor1, packed, lane);
+  if constexpr (P::LO8) conv3_lo_pass<P, L>(smem, packed, tail, lor0, lor1, ci, h, lane, acc);
   preload_ring<kRing, kCoutArr[L + 1] / 32>(next, layer_weights<P, L + 1>(packed, lane));
   C6_MARK(4 + 2 * L);
   finish_layer<P, NT>(smem, ci, h, acc, [] {});
@@ -642,8 +768,11 @@ __global__ __launch_bounds__(256) void fused_forward_kernel(const FwdParams prm)
       const float *valw = polw + kHeadC;
       const float *pwl = polw + 4 * h;  // per-lane base: channel 32t + 8q + 4h + e
       asm volatile("" : "+v"(pwl));
+      v4i lor0[LoRing<P, 7>::D][LoRing<P, 7>::NT], lor1[LoRing<P, 7>::D][LoRing<P, 7>::NT];
       conv3_pass<P, 96, 96>(smem, layer_weights<P, 7>(packed, lane), r8, ci, h, acc);
-      if constexpr (P::LO8) conv3_lo_pass<P, 7>(smem, packed, tail, ci, h, lane, acc);
+      C6_MARK(37);
+      if constexpr (P::LO8) lo_preload<P, 7>(lor0, lor1, packed, lane);
+      if constexpr (P::LO8) conv3_lo_pass<P, 7>(smem, packed, tail, lor0, lor1, ci, h, lane, acc);
       if (bn < prm.total_boards) preload_ring<L1Pipe<P>::D, 1>(r1, layer_weights<P, 0>(packed_of(bn), lane));
       C6_MARK(18);
       float pol[3] = {0.0f, 0.0f, 0.0f};
@@ -750,6 +879,20 @@ template <class P> __global__ void pack_kernel(const PackParams prm) {
             const int tap = g / per32, cb = g % per32, co = 32 * t + m;
             const float *w = prm.conv_w[ll];
             const float sc = exp2f((float)reinterpret_cast<const int *>(prm.packed + G::TAIL_OFF)[G::TAIL_SW + ll]);
+            if constexpr (P::LO6) {  // the lane's 32 K slots as e2m3: 24 bytes = piece 0 + half of piece 1
+              f32x16v even, odd;
+#pragma unroll
+              for (int i = 0; i < 16; ++i) {
+                even[i] = (float)(__bf16)w[(co * cin + lo6_channel(cin, cb, 2 * i)) * 9 + tap] * sc;
+                odd[i] = (float)(__bf16)w[(co * cin + lo6_channel(cin, cb, 2 * i + 1)) * 9 + tap] * sc;
+              }
+              const u32x6 r = to_fp6_block(even, odd, 1.0f);
+              if (piece == 0) {
+                o = v4i{(int)r[0], (int)r[1], (int)r[2], (int)r[3]};
+              } else {
+                o = v4i{(int)r[4], (int)r[5], 0, 0};
+              }
+            } else
 #pragma unroll
             for (int d = 0; d < 4; ++d) {
               float v[4];
@@ -816,7 +959,8 @@ template <class P> __global__ void pack_kernel(const PackParams prm) {
   }
 }
 
-// sw[l] = largest power of two that keeps 2^sw * max|w_l| inside e4m3's range (one block per layer)
+// sw[l] = largest power of two that keeps 2^sw * max|w_l| inside the range of the low-order
+// weight copy's format (one block per layer)
 template <class P> __global__ __launch_bounds__(256) void lo_scale_kernel(const PackParams prm) {
   using G = Geo<P>;
   __shared__ float red[256];
@@ -837,7 +981,8 @@ template <class P> __global__ __launch_bounds__(256) void lo_scale_kernel(const 
   }
   if (threadIdx.x == 0) {
     int e = 0;
-    if (red[0] > 0.0f && red[0] < INFINITY) e = (int)floorf(log2f(448.0f / red[0]));
+    constexpr float kLargest = P::LO6 ? 7.5f : 448.0f;  // of e2m3 / e4m3
+    if (red[0] > 0.0f && red[0] < INFINITY) e = (int)floorf(log2f(kLargest / red[0]));
     sw[l] = e < -20 ? -20 : (e > 20 ? 20 : e);
   }
 }
@@ -899,6 +1044,7 @@ int dispatch_pack(int prec, const PackParams &pp, hipStream_t st) {
     case C6_PREC_F16: return launch_pack<PrecF16>(pp, st);
     case C6_PREC_BF16X2: return launch_pack<PrecBF16X2>(pp, st);
     case C6_PREC_BF16F8: return launch_pack<PrecBF16F8>(pp, st);
+    case C6_PREC_BF16F6: return launch_pack<PrecBF16F6>(pp, st);
   }
   set_error("unknown precision mode %d", prec);
   return C6_EINVAL;
@@ -911,6 +1057,7 @@ int dispatch_forward(int prec, const FwdParams &fp, hipStream_t st) {
     case C6_PREC_F16: return launch_forward<PrecF16>(fp, st);
     case C6_PREC_BF16X2: return launch_forward<PrecBF16X2>(fp, st);
     case C6_PREC_BF16F8: return launch_forward<PrecBF16F8>(fp, st);
+    case C6_PREC_BF16F6: return launch_forward<PrecBF16F6>(fp, st);
   }
   set_error("unknown precision mode %d", prec);
   return C6_EINVAL;
@@ -923,6 +1070,7 @@ size_t packed_bytes(int prec) {
     case C6_PREC_F16: return Geo<PrecF16>::PACKED_BYTES;
     case C6_PREC_BF16X2: return Geo<PrecBF16X2>::PACKED_BYTES;
     case C6_PREC_BF16F8: return Geo<PrecBF16F8>::PACKED_BYTES;
+    case C6_PREC_BF16F6: return Geo<PrecBF16F6>::PACKED_BYTES;
   }
   return 0;
 }

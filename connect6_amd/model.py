@@ -199,8 +199,9 @@ class PolicyValueNet(nn.Module):
     PyTorch's own rules (bf16/fp16 under ``torch.autocast`` or when the
     parameters are held in that dtype, else fp32); or one of ``"fp32"``,
     ``"bf16"``, ``"fp16"``, ``"bf16x2"`` (bf16 MFMA with activations carried
-    as a hi+lo bf16 pair), ``"bf16f8"`` (bf16 MFMA plus a correction pass on
-    the activations' low-order part held in fp8).
+    as a hi+lo bf16 pair), ``"bf16f8"`` / ``"bf16f6"`` (bf16 MFMA plus a
+    correction pass on the activations' low-order part held in fp8 / in
+    block-scaled fp6).
     """
 
     DEFAULT_KERNELS = (23, 3, 3, 3, 3, 3, 3, 3)

@@ -37,6 +37,8 @@ extern "C" {
 #define C6_PREC_BF16X2 3 /* bf16 MFMA, activations carried as a bf16 hi+lo pair (two passes)  */
 #define C6_PREC_BF16F8 4 /* bf16 MFMA + a second pass on the activations' dropped low-order
                             part held as scaled fp8 (e4m3), on the fp8 MFMA at twice the rate */
+#define C6_PREC_BF16F6 5 /* the same with the low-order part held as block-scaled fp6 (e2m3,
+                            one power-of-two scale per 32 channels), at four times the rate */
 
 /* element types of caller tensors */
 #define C6_DT_F32 0

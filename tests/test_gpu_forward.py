@@ -69,7 +69,7 @@ def test_zero_input_known_answer(cuda):
     # reference init (zero biases) every logit and the value are exactly zero
     model = c6.PolicyValueNet(board_size=19).to(cuda)
     with torch.inference_mode():
-        for prec in (None, "bf16", "fp16", "bf16x2", "bf16f8"):
+        for prec in (None, "bf16", "fp16", "bf16x2", "bf16f8", "bf16f6"):
             model.precision = prec
             logits, value = model(torch.zeros(3, 3, 19, 19, device=cuda))
             assert logits.shape == (3, 361) and value.shape == (3,)
@@ -94,7 +94,7 @@ def test_empty_batch(cuda):
 
 
 @pytest.mark.parametrize("init", ["reference", "torch_default"])
-@pytest.mark.parametrize("prec", ["bf16f8", "bf16x2", "fp16", "bf16"])
+@pytest.mark.parametrize("prec", ["bf16f6", "bf16f8", "bf16x2", "fp16", "bf16"])
 def test_16bit_paths_match_fp32_oracle_b4096(cuda, oracle_cfg2, init, prec):
     x, legal, outs = oracle_cfg2
     st, lo, vo = outs[init]
@@ -158,7 +158,7 @@ def test_grad_mode_is_refused(cuda):
         model(torch.zeros(1, 3, 19, 19, device=cuda))
 
 
-@pytest.mark.parametrize("prec", [None, "bf16x2", "bf16f8"])
+@pytest.mark.parametrize("prec", [None, "bf16x2", "bf16f8", "bf16f6"])
 def test_masking_is_bit_exact(cuda, prec):
     st = R.init_state(1234, "reference")
     x, legal = gen_boards(512, 200, 2025)
@@ -214,7 +214,7 @@ def test_grouped_fp32_matches_individual_models(cuda):
     assert rel_l2(grouped, ref) <= FP32_TOL
 
 
-@pytest.mark.parametrize("precision", [None, "bf16x2", "bf16f8"])
+@pytest.mark.parametrize("precision", [None, "bf16x2", "bf16f8", "bf16f6"])
 def test_grouped_g8_bf16_cfg3(cuda, precision):
     torch.set_num_threads(16)
     cps = _checkpoints(8)
@@ -269,7 +269,7 @@ def test_runs_on_the_callers_stream_and_accepts_strided_input(cuda):
         assert torch.equal(got, want) and torch.equal(vgot, vwant)
 
 
-@pytest.mark.parametrize("prec", ["bf16f8", "bf16x2", "bf16", "fp16"])
+@pytest.mark.parametrize("prec", ["bf16f6", "bf16f8", "bf16x2", "bf16", "fp16"])
 def test_large_activations_stay_finite(cuda, prec):
     # weights 6x larger per layer: activations reach the hundreds, far beyond what the fp8 low-order
     # plane can represent (its inputs are clamped, so accuracy degrades to bf16's, never to NaN)

@@ -183,7 +183,7 @@ def test_forward_from_board_states(cuda, view):
     assert torch.equal(lg, same) and torch.equal(vg, vsame)
     # whole batch, no gather, with the fused draw
     u = gen_uniform(300, 2)
-    model.precision = "bf16f8"
+    model.precision = "bf16f6"
     with torch.inference_mode():
         a, lp, v = model.selfplay_step_boards(boards.to(cuda), player.to(cuda), left.to(cuda), u.to(cuda),
                                               0.9, view=view)

@@ -42,6 +42,7 @@ def test_packed_sizes_follow_the_layout():
     for cin, cout in zip((32, 32, 64, 64, 64, 96, 96), (32, 64, 64, 64, 96, 96, 96)):
         lo += ((9 * cin // 32 + 1) // 2) * (cout // 32) * 2
     assert _lib.packed_bytes(_lib.PREC_BF16F8) == (frags(8) + lo + 18) * 1024 + tail
+    assert _lib.packed_bytes(_lib.PREC_BF16F6) == _lib.packed_bytes(_lib.PREC_BF16F8)  # same fragment grid
     with pytest.raises(ValueError):
         _lib.packed_bytes(9)
 
