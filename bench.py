@@ -230,6 +230,33 @@ def main() -> int:
         hbm["d4_expand_f32"] = {"GBps": nd * 3 * 361 * 4 * 9 / t / 1e9, "boards": nd}
         t = event_timed(lambda: c6.d4_reduce(views, vals))
         hbm["d4_reduce"] = {"GBps": nd * (361 * 4 * 9 + 4 * 9) / t / 1e9, "boards": nd}
+        # environment step (VectorConnect6.step) and canonical input on mid-game positions
+        xe, le = gen_boards(nb, 200, 11)
+        env = c6.VectorConnect6(nb, 19, 6, device=dev)
+        env.boards.copy_((xe[:, 0] - xe[:, 1]).to(torch.int8))
+        env.empty_count.copy_(le.sum(1).to(torch.int16))
+        env.move_count.copy_((361 - le.sum(1)).to(torch.int16))
+        acts = torch.rand(le.shape).masked_fill(~le, -1.0).argmax(1).to(dev)
+        t = event_timed(lambda: env.step(acts))
+        # per game: action 8 + state 6 + up to 40 neighbour squares in; stone 1 + state 6 + results 9 out
+        hbm["env_step"] = {"GBps": nb * 70 / t / 1e9, "boards": nb, "games_per_s": nb / t}
+        t = event_timed(lambda: env.network_input())
+        hbm["canonical_input"] = {"GBps": nb * (361 + 2 + 3 * 361 * 4) / t / 1e9, "boards": nb}
+        env16 = c6.VectorConnect6(16384, 19, 6, device=dev)
+        env16.boards.copy_(env.boards[:16384])
+        t16 = event_timed(lambda: env16.step(acts[:16384]))
+        out["env_step_b16384"] = {"games_per_s": 16384 / t16, "us": t16 * 1e6}
+        # one whole collector iteration (connect6/train.py:730-748, :791-799, :854-864 of the
+        # reference): int8 state -> view -> forward -> mask -> sample -> map back -> step -> reset
+        def collector_iteration():
+            a_, _, _ = model.selfplay_step_boards(env16.boards, env16.current_player, env16.stones_left,
+                                                  us, 1.0, view=5)
+            step = env16.step(a_, view=5)
+            env16.reset(torch.nonzero(step.done).flatten())
+        env16.reset()
+        tc = timed(collector_iteration, steps=20)
+        out["collector_iteration_b16384"] = {"boards_per_s": 16384 / tc, "ms": tc * 1e3}
+        del env, env16, xe, le, acts
         for v in hbm.values():
             v["frac_of_hbm_peak"] = v["GBps"] / HBM_PEAK_GBS
         out["hbm_kernels"] = hbm

@@ -1,8 +1,8 @@
 """connect6_amd: the Connect6 policy/value CNN forward path on MI355X (gfx950).
 
 Host-side mirror of the reference's operator interface for this path
-(connect6/model.py and connect6/history.py:186-303) over a C-ABI library of
-hand-written HIP kernels.
+(connect6/model.py, connect6/history.py:186-303 and connect6/vector_env.py) over
+a C-ABI library of hand-written HIP kernels.
 """
 from ._lib import C6Error, build, load
 from .history import HistoricalCheckpoint, HistoricalPolicyEnsemble
@@ -17,14 +17,19 @@ from .selfplay import (
     transform_actions,
     transform_boards,
 )
+from .vector_env import StepBatch, VectorConnect6, canonical_network_input, canonical_observation
 
 __all__ = [
     "C6Error",
     "HistoricalCheckpoint",
     "HistoricalPolicyEnsemble",
     "PolicyValueNet",
+    "StepBatch",
+    "VectorConnect6",
     "build",
     "build_model",
+    "canonical_network_input",
+    "canonical_observation",
     "d4_expand",
     "d4_reduce",
     "evaluate_d4",

@@ -14,7 +14,7 @@ _PKG = Path(__file__).resolve().parent
 _CSRC = _PKG / "csrc"
 _LIBDIR = _PKG / "lib"
 _SO = _LIBDIR / "libconnect6_amd.so"
-_SOURCES = ("c6_forward.hip", "c6_tail.hip", "c6_generic.hip", "c6_api.hip")
+_SOURCES = ("c6_forward.hip", "c6_tail.hip", "c6_generic.hip", "c6_env.hip", "c6_api.hip")
 
 # arithmetic modes (include/connect6_amd.h)
 PREC_F32, PREC_BF16, PREC_F16, PREC_BF16X2, PREC_BF16F8, PREC_BF16F6 = 0, 1, 2, 3, 4, 5
@@ -37,6 +37,8 @@ EXPORTS = (
     "c6_softmax_sample",
     "c6_d4_expand",
     "c6_d4_reduce",
+    "c6_env_step",
+    "c6_canonical_input",
 )
 
 
@@ -107,6 +109,10 @@ def load() -> ctypes.CDLL:
     lib.c6_d4_expand.argtypes = [vp, i32, i64, vp, vp]
     lib.c6_d4_reduce.restype = i32
     lib.c6_d4_reduce.argtypes = [vp, vp, i64, vp, vp, vp]
+    lib.c6_env_step.restype = i32
+    lib.c6_env_step.argtypes = [vp, vp, vp, vp, vp, vp, i32, i64, i32, i32, vp, vp, vp, vp, vp, vp]
+    lib.c6_canonical_input.restype = i32
+    lib.c6_canonical_input.argtypes = [vp, vp, vp, i64, i32, vp, vp]
     _lib = lib
     return lib
 

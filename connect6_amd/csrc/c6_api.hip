@@ -32,6 +32,10 @@ int launch_generic(const void *x, int x_dtype, long long batch, int n, int layer
                    float *logits, float *value, int mask_mode, const uint8_t *legal, float fill,
                    hipStream_t st);
 
+int launch_env_step(const EnvParams &p, hipStream_t st);
+int launch_canonical_input(const int8_t *boards, const int8_t *player, const int8_t *stones_left,
+                           long long num, int n, float *out, hipStream_t st);
+
 static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 static int elem_bytes(int dt) { return dt == C6_DT_F32 ? 4 : ((dt == C6_DT_BF16 || dt == C6_DT_F16) ? 2 : 0); }
 static bool valid_prec(int p) { return p >= C6_PREC_F32 && p <= C6_PREC_BF16F6; }
@@ -308,6 +312,55 @@ int c6_softmax_sample(const float *logits, const uint8_t *legal, const float *u,
   const float inv_t = 1.0f / (temperature > 1e-4f ? temperature : 1e-4f);
   return launch_sample(logits, legal, u, inv_t, batch, reinterpret_cast<long long *>(actions),
                        logprob, static_cast<hipStream_t>(stream));
+}
+
+int c6_env_step(int8_t *boards, int8_t *current_player, int8_t *stones_left, int16_t *empty_count,
+                int16_t *move_count, const int64_t *actions, int view, int64_t num_envs,
+                int board_size, int win_length, float *reward, uint8_t *done, int8_t *winner,
+                int8_t *transition_sign, int16_t *game_lengths, void *stream) {
+  if (num_envs < 0 || board_size < 1 || board_size > 181 || win_length < 1 || view < 0 || view > 7) {
+    set_error("c6_env_step: bad sizes (num_envs %lld, board_size %d, win_length %d) or view %d",
+              (long long)num_envs, board_size, win_length, view);
+    return C6_EINVAL;
+  }
+  if (num_envs > 0 && (!boards || !current_player || !stones_left || !empty_count || !move_count ||
+                       !actions || !reward || !done || !winner || !transition_sign || !game_lengths)) {
+    set_error("c6_env_step: null state, action or result pointer");
+    return C6_EINVAL;
+  }
+  EnvParams p;
+  p.boards = boards;
+  p.player = current_player;
+  p.stones_left = stones_left;
+  p.empty_count = empty_count;
+  p.move_count = move_count;
+  p.actions = reinterpret_cast<const long long *>(actions);
+  p.num = num_envs;
+  p.n = board_size;
+  p.win = win_length;
+  p.view = view;
+  p.reward = reward;
+  p.done = done;
+  p.winner = winner;
+  p.sign = transition_sign;
+  p.lengths = game_lengths;
+  return launch_env_step(p, static_cast<hipStream_t>(stream));
+}
+
+int c6_canonical_input(const int8_t *boards, const int8_t *current_player,
+                       const int8_t *stones_left, int64_t num_envs, int board_size, float *out,
+                       void *stream) {
+  if (num_envs < 0 || board_size < 1 || board_size > 181) {
+    set_error("c6_canonical_input: bad sizes (num_envs %lld, board_size %d)", (long long)num_envs,
+              board_size);
+    return C6_EINVAL;
+  }
+  if (num_envs > 0 && (!boards || !current_player || !stones_left || !out)) {
+    set_error("c6_canonical_input: null pointer");
+    return C6_EINVAL;
+  }
+  return launch_canonical_input(boards, current_player, stones_left, num_envs, board_size, out,
+                                static_cast<hipStream_t>(stream));
 }
 
 int c6_d4_expand(const void *x, int dtype, int64_t batch, void *out, void *stream) {

@@ -214,6 +214,23 @@ struct PackParams {
   unsigned char *packed;
 };
 
+// state and results of VectorConnect6.step (connect6/vector_env.py:33-53, :8-14 of the reference)
+struct EnvParams {
+  int8_t *boards;        // [N, n, n]
+  int8_t *player;        // [N]
+  int8_t *stones_left;   // [N]
+  int16_t *empty_count;  // [N]
+  int16_t *move_count;   // [N]
+  const long long *actions;
+  long long num;
+  int n, win;
+  int view;              // actions are squares of D4 view `view` of the board (0 = the board itself)
+  float *reward;
+  uint8_t *done;
+  int8_t *winner, *sign;
+  int16_t *lengths;
+};
+
 void set_error(const char *fmt, ...);
 
 }  // namespace c6

@@ -98,8 +98,8 @@ __device__ __forceinline__ int d4_to_view(int a, int p) {
   return rr * n + cc;
 }
 // square v of view p -> canonical square (connect6/train.py:256-277)
-__device__ __forceinline__ int d4_from_view(int v, int p) {
-  const int n = kBoard, k = p & 3;
+__device__ __forceinline__ int d4_from_view(int v, int p, int n = kBoard) {
+  const int k = p & 3;
   int r = v / n, c = v - r * n;
   if (p >= 4) c = n - 1 - c;
   int rr = r, cc = c;

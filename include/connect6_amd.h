@@ -161,6 +161,34 @@ int c6_d4_expand(const void *x, int dtype, int64_t batch, void *out, void *strea
 int c6_d4_reduce(const float *view_logits, const float *view_values, int64_t batch,
                  float *logits, float *values, void *stream);
 
+/* One step of N Connect6 games held as device tensors.
+ * Replaces: VectorConnect6.step and _check_win_local (connect6/vector_env.py:106-193).
+ * State, updated in place (layouts of connect6/vector_env.py:33-53):
+ *   boards int8 [N,n,n] (+1 / -1 / 0), current_player int8 [N], stones_left int8 [N],
+ *   empty_count int16 [N], move_count int16 [N]
+ * actions int64 [N]: square row*n + col each game plays (values outside [0, n*n) are clamped;
+ *   like the reference without debug_checks, an occupied square is overwritten).
+ * view: 0, or the D4 view 1..7 (numbering of _symmetry_for_phase) the actions are expressed
+ *   in; they are mapped back as _inverse_transform_actions does (connect6/train.py:256-277,
+ *   :854-862) before the stone is placed.
+ * Results (connect6/vector_env.py:8-14, StepBatch): reward fp32 [N] (1 if the move made a line
+ * of win_length or more), done uint8/bool [N] (win, or board full), winner int8 [N],
+ * transition_sign int8 [N] (+1 same side moves again, -1 side changed, 0 game over),
+ * game_lengths int16 [N] (= move_count after the move).  A finished game keeps its side to
+ * move and stones_left; the caller resets it. */
+int c6_env_step(int8_t *boards, int8_t *current_player, int8_t *stones_left, int16_t *empty_count,
+                int16_t *move_count, const int64_t *actions, int view, int64_t num_envs,
+                int board_size, int win_length, float *reward, uint8_t *done, int8_t *winner,
+                int8_t *transition_sign, int16_t *game_lengths, void *stream);
+
+/* Network input planes of N games.
+ * Replaces: canonical_network_input (connect6/vector_env.py:196-218).
+ * out fp32 [N,3,n,n]: plane 0 = boards == current_player, plane 1 = boards == -current_player,
+ * plane 2 = stones_left == 1 (broadcast over the board). */
+int c6_canonical_input(const int8_t *boards, const int8_t *current_player,
+                       const int8_t *stones_left, int64_t num_envs, int board_size, float *out,
+                       void *stream);
+
 #ifdef __cplusplus
 }
 #endif

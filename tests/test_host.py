@@ -68,6 +68,14 @@ def test_entry_points_reject_bad_arguments_before_touching_the_device():
                                  None, None, None) == -1
     assert lib.c6_forward_boards(None, None, None, 4, None, 0, 0, None, 1, None, None, 1, 0.0, None, 1.0,
                                  None, None, None) == 0
+    none14 = [None] * 5
+    assert lib.c6_env_step(*none14, None, 0, 4, 19, 6, None, None, None, None, None, None) == -1  # null state
+    assert lib.c6_env_step(*none14, None, 0, 4, 0, 6, None, None, None, None, None, None) == -1   # board size
+    assert lib.c6_env_step(*none14, None, 0, 4, 19, 0, None, None, None, None, None, None) == -1  # win length
+    assert lib.c6_env_step(*none14, None, 8, 4, 19, 6, None, None, None, None, None, None) == -1  # view
+    assert lib.c6_env_step(*none14, None, 0, 0, 19, 6, None, None, None, None, None, None) == 0   # no games
+    assert lib.c6_canonical_input(None, None, None, 3, 19, None, None) == -1
+    assert lib.c6_canonical_input(None, None, None, 0, 19, None, None) == 0
     n = ctypes.c_size_t(0)
     ch = (ctypes.c_int * 3)(8, 8, 16)
     ks = (ctypes.c_int * 3)(3, 3, 3)
@@ -243,3 +251,13 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
         _lib.load()
     with pytest.raises(c6.C6Error):
         _lib.packed_bytes(_lib.PREC_BF16)
+
+
+def test_vector_env_refuses_cpu_device():
+    import connect6_amd as c6
+
+    with pytest.raises(RuntimeError, match="HIP device only"):
+        c6.VectorConnect6(4, 9, 6, device="cpu")
+    with pytest.raises(RuntimeError, match="HIP device"):
+        c6.canonical_network_input(torch.zeros(1, 9, 9, dtype=torch.int8), torch.ones(1, dtype=torch.int8),
+                                   torch.ones(1, dtype=torch.int8))
