@@ -593,7 +593,10 @@ __device__ __forceinline__ void mid_layer(
   C6_MARK(30 + L);
   if constexpr (P::LO8) lo_preload<P, L>(lor0, lor1, packed, lane);
   if constexpr (P::LO8) conv3_lo_pass<P, L>(smem, packed, tail, lor0, lor1, ci, h, lane, acc);
-  preload_ring<kRing, kCoutArr[L + 1] / 32>(next, layer_weights<P, L + 1>(packed, lane));
+  // With equal channel counts the main pass's over-read has already left the next layer's first
+  // kRing k-steps in the ring (same fragment order, contiguous in memory): `next` is `ring`.
+  if constexpr (kCoutArr[L + 1] != kCoutArr[L])
+    preload_ring<kRing, kCoutArr[L + 1] / 32>(next, layer_weights<P, L + 1>(packed, lane));
   C6_MARK(4 + 2 * L);
   finish_layer<P, NT>(smem, ci, h, acc, [] {});
   C6_MARK(5 + 2 * L);
@@ -732,8 +735,7 @@ __global__ __launch_bounds__(256) void fused_forward_kernel(const FwdParams prm)
     __syncthreads();
     C6_MARK(1);
 
-    v4i r2[kRing][1], r3[kRing][2], r4[kRing][2], r5[kRing][2], r6[kRing][3], r7[kRing][3],
-        r8[kRing][3];
+    v4i r2[kRing][1], r345[kRing][2], r678[kRing][3];  // weight rings of layers 2, 3-5, 6-8
     // ---- layer 1 ----
     {
       f32x16 acc[1][3];
@@ -753,12 +755,12 @@ __global__ __launch_bounds__(256) void fused_forward_kernel(const FwdParams prm)
       });
     }
     C6_MARK(3);
-    mid_layer<P, 1>(smem, packed, tail, r2, r3, ci, h, lane, wave, trace_on);
-    mid_layer<P, 2>(smem, packed, tail, r3, r4, ci, h, lane, wave, trace_on);
-    mid_layer<P, 3>(smem, packed, tail, r4, r5, ci, h, lane, wave, trace_on);
-    mid_layer<P, 4>(smem, packed, tail, r5, r6, ci, h, lane, wave, trace_on);
-    mid_layer<P, 5>(smem, packed, tail, r6, r7, ci, h, lane, wave, trace_on);
-    mid_layer<P, 6>(smem, packed, tail, r7, r8, ci, h, lane, wave, trace_on);
+    mid_layer<P, 1>(smem, packed, tail, r2, r345, ci, h, lane, wave, trace_on);
+    mid_layer<P, 2>(smem, packed, tail, r345, r345, ci, h, lane, wave, trace_on);
+    mid_layer<P, 3>(smem, packed, tail, r345, r345, ci, h, lane, wave, trace_on);
+    mid_layer<P, 4>(smem, packed, tail, r345, r678, ci, h, lane, wave, trace_on);
+    mid_layer<P, 5>(smem, packed, tail, r678, r678, ci, h, lane, wave, trace_on);
+    mid_layer<P, 6>(smem, packed, tail, r678, r678, ci, h, lane, wave, trace_on);
 
     // ---- layer 8 + both 1x1 heads straight from the fp32 accumulators ----
     {
@@ -769,7 +771,7 @@ __global__ __launch_bounds__(256) void fused_forward_kernel(const FwdParams prm)
       const float *pwl = polw + 4 * h;  // per-lane base: channel 32t + 8q + 4h + e
       asm volatile("" : "+v"(pwl));
       v4i lor0[LoRing<P, 7>::D][LoRing<P, 7>::NT], lor1[LoRing<P, 7>::D][LoRing<P, 7>::NT];
-      conv3_pass<P, 96, 96>(smem, layer_weights<P, 7>(packed, lane), r8, ci, h, acc);
+      conv3_pass<P, 96, 96>(smem, layer_weights<P, 7>(packed, lane), r678, ci, h, acc);
       C6_MARK(37);
       if constexpr (P::LO8) lo_preload<P, 7>(lor0, lor1, packed, lane);
       if constexpr (P::LO8) conv3_lo_pass<P, 7>(smem, packed, tail, lor0, lor1, ci, h, lane, acc);
