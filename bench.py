@@ -25,6 +25,10 @@ if str(ROOT) not in sys.path:
 CONV_FLOP_PER_BOARD = 269_554_368        # dense conv count, 2 * 134,777,184 MAC
 MFMA_PEAK_TFLOPS = 2500.0                # MI355X dense bf16 / fp16
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per B=4096 launch of the fused kernel: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (one
+# run each), scaled by what the same counters read for a 256 MiB copy (x2.00 and x1.00); the
+# figures and commands are in profiles/fused_forward_<mode>_b4096.md.
+TRAFFIC_BYTES = {"bf16f6": 39.3e6, "bf16f8": 45.6e6, "bf16": 35.8e6}
 HEADLINE = "bf16f6"                      # fastest bf16-MFMA mode that meets the >= 99 % argmax gate
 
 
@@ -112,7 +116,8 @@ def main() -> int:
             "peak": MFMA_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": achieved / MFMA_PEAK_TFLOPS,
-            "traffic": None,
+            "traffic": TRAFFIC_BYTES.get(args.precision),
+            "traffic_unit": "bytes per launch",
             "kernel": "fused_forward_kernel",
             "kernel_ms": kern * 1e3,
             "flop_per_board": CONV_FLOP_PER_BOARD,
