@@ -681,20 +681,29 @@ __global__ __launch_bounds__(256) void fused_forward_kernel(const FwdParams prm)
     }
   };
 
-  long long b = blockIdx.x;
-  if (b >= prm.total_boards) return;
+  // Each workgroup takes one contiguous run of boards, and the runs are dealt out so that the
+  // workgroups of one XCD (workgroup i runs on XCD i % 8) cover one contiguous eighth of the
+  // batch: with several weight sets an XCD's L2 then holds only the sets of its own boards, and
+  // consecutive boards of a workgroup mostly reuse the set it has just streamed.
+  const long long per = (prm.total_boards + gridDim.x - 1) / gridDim.x;
+  const unsigned xcds = (gridDim.x % 8 == 0) ? 8 : 1;
+  const long long run = (long long)(blockIdx.x % xcds) * (gridDim.x / xcds) + blockIdx.x / xcds;
+  long long b = run * per;
+  const long long b_end = b + per < prm.total_boards ? b + per : prm.total_boards;
+  if (b >= b_end) return;
+  [[maybe_unused]] const long long b_first = b;
   v4i r1[L1Pipe<P>::D][1];
   preload_ring<L1Pipe<P>::D, 1>(r1, layer_weights<P, 0>(packed_of(b), lane));
   fetch_board(b);
 
-  for (; b < prm.total_boards; b += gridDim.x) {
+  for (; b < b_end; ++b) {
     int tidv = tid;  // opaque per board: keeps per-thread staging addresses out of long-lived registers
     asm volatile("" : "+v"(tidv));
     const unsigned char *packed = packed_of(b);
     const float *tail = reinterpret_cast<const float *>(packed + G::TAIL_OFF);
 
 #ifdef C6_TRACE
-    const bool trace_on = (b == blockIdx.x + 2LL * gridDim.x);  // third board of this workgroup
+    const bool trace_on = (b == b_first + 2);  // third board of this workgroup
 #else
     const bool trace_on = false;
 #endif
@@ -730,8 +739,8 @@ __global__ __launch_bounds__(256) void fused_forward_kernel(const FwdParams prm)
         }
       }
     }
-    const long long bn = b + gridDim.x;
-    if (bn < prm.total_boards) fetch_board(bn);  // lands while this board is computed
+    const long long bn = b + 1;
+    if (bn < b_end) fetch_board(bn);  // lands while this board is computed
     __syncthreads();
     C6_MARK(1);
 
@@ -775,7 +784,7 @@ __global__ __launch_bounds__(256) void fused_forward_kernel(const FwdParams prm)
       C6_MARK(37);
       if constexpr (P::LO8) lo_preload<P, 7>(lor0, lor1, packed, lane);
       if constexpr (P::LO8) conv3_lo_pass<P, 7>(smem, packed, tail, lor0, lor1, ci, h, lane, acc);
-      if (bn < prm.total_boards) preload_ring<L1Pipe<P>::D, 1>(r1, layer_weights<P, 0>(packed_of(bn), lane));
+      if (bn < b_end) preload_ring<L1Pipe<P>::D, 1>(r1, layer_weights<P, 0>(packed_of(bn), lane));
       C6_MARK(18);
       float pol[3] = {0.0f, 0.0f, 0.0f};
       float vsum = 0.0f;
