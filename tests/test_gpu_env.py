@@ -185,3 +185,18 @@ def test_collector_loop_plays_legal_games_to_the_end(cuda):
             assert bool(torch.isfinite(logprob).all()) and bool(value.abs().le(1).all())
     assert finished > 0
     assert bool((env.boards.ne(0).flatten(1).sum(1).to(torch.int16) == env.move_count).all())
+
+
+def test_committed_env_rollout(cuda):
+    import numpy as np
+    from pathlib import Path
+
+    g = np.load(Path(__file__).resolve().parent / "golden" / "env_rollout_golden.npz")
+    env = c6.VectorConnect6(48, 19, 6, device=cuda)
+    for i in range(g["actions"].shape[0]):
+        out = env.step(torch.from_numpy(g["actions"][i]).to(cuda))
+        for k in ("reward", "done", "winner", "transition_sign", "game_lengths"):
+            assert np.array_equal(getattr(out, k).cpu().numpy(), g[k][i]), (k, i)
+        env.reset(torch.nonzero(out.done).flatten())
+    for k in ("boards", "current_player", "stones_left", "empty_count", "move_count"):
+        assert np.array_equal(getattr(env, k).cpu().numpy(), g[k])

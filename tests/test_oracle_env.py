@@ -104,3 +104,18 @@ def test_draw_on_board_without_room_for_a_line():
 def test_bad_action_shape_raises():
     with pytest.raises(ValueError):
         E.step(E.new_state(4, 9, 6), torch.zeros(3, dtype=torch.long))
+
+
+def test_oracle_reproduces_committed_env_rollout():
+    from pathlib import Path
+
+    g = np.load(Path(__file__).resolve().parent / "golden" / "env_rollout_golden.npz")
+    st = E.new_state(48, 19, 6)
+    for i in range(g["actions"].shape[0]):
+        out = E.step(st, torch.from_numpy(g["actions"][i]))
+        for k in ("reward", "done", "winner", "transition_sign", "game_lengths"):
+            assert np.array_equal(getattr(out, k).numpy(), g[k][i]), (k, i)
+        E.reset(st, torch.nonzero(out.done).flatten())
+    for k in ("boards", "current_player", "stones_left", "empty_count", "move_count"):
+        assert np.array_equal(getattr(st, k).numpy(), g[k])
+    assert g["done"].sum() >= 50 and g["reward"].sum() >= 50      # the fixture holds real wins
