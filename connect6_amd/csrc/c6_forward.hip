@@ -545,16 +545,22 @@ __device__ __forceinline__ void store_tile_lo6(unsigned char *smem, int pos_in, 
   }
 }
 
+typedef const __attribute__((address_space(1))) float *GlobalF32;
+typedef const __attribute__((address_space(1))) f32x4 *GlobalF32x4;
+
 // accumulators start at the layer's bias: lane (h) register i holds channel 32t + 8(i/4) + 4h + i%4
 template <int N>
 __device__ __forceinline__ void init_acc(f32x16 (&acc)[N][3], const float *__restrict__ bias, int h) {
-  const float *bl = bias + 4 * h;  // one per-lane base; every load below is base + constant
-  asm volatile("" : "+v"(bl));
+  const float *blg = bias + 4 * h;  // one per-lane base; every load below is base + constant
+  asm volatile("" : "+v"(blg));
+  // (the laundering hides that this is global memory; say so again, or the loads become flat
+  // loads, which also count against the LDS counter)
+  const GlobalF32 bl = (GlobalF32)blg;
 #pragma unroll
   for (int t = 0; t < N; ++t)
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      const f32x4 b4 = *reinterpret_cast<const f32x4 *>(bl + 32 * t + 8 * q);
+      const f32x4 b4 = *(GlobalF32x4)(bl + 32 * t + 8 * q);
 #pragma unroll
       for (int j = 0; j < 3; ++j)
 #pragma unroll
@@ -779,6 +785,7 @@ __global__ __launch_bounds__(256) void fused_forward_kernel(const FwdParams prm)
       const float *valw = polw + kHeadC;
       const float *pwl = polw + 4 * h;  // per-lane base: channel 32t + 8q + 4h + e
       asm volatile("" : "+v"(pwl));
+      const GlobalF32 pwg = (GlobalF32)pwl;
       v4i lor0[LoRing<P, 7>::D][LoRing<P, 7>::NT], lor1[LoRing<P, 7>::D][LoRing<P, 7>::NT];
       conv3_pass<P, 96, 96>(smem, layer_weights<P, 7>(packed, lane), r678, ci, h, acc);
       C6_MARK(37);
@@ -792,8 +799,8 @@ __global__ __launch_bounds__(256) void fused_forward_kernel(const FwdParams prm)
       for (int t = 0; t < 3; ++t)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const f32x4 pw = *reinterpret_cast<const f32x4 *>(pwl + 32 * t + 8 * q);
-          const f32x4 vw = *reinterpret_cast<const f32x4 *>(pwl + kHeadC + 32 * t + 8 * q);
+          const f32x4 pw = *(GlobalF32x4)(pwg + 32 * t + 8 * q);
+          const f32x4 vw = *(GlobalF32x4)(pwg + kHeadC + 32 * t + 8 * q);
 #pragma unroll
           for (int j = 0; j < 3; ++j) {
             float vs = 0.0f;
