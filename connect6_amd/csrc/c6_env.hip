@@ -65,23 +65,62 @@ __global__ __launch_bounds__(256) void env_step_kernel(const EnvParams p) {
   p.sign[i] = sign;
 }
 
-// one thread per board cell: plane 0 = stone of the side to move, 1 = of the other side,
-// 2 = this decision is the last stone of the turn.  (A variant with one 16-byte store per thread
-// measured slower: its byte loads stop being coalesced.)
+// Plane 0 = stone of the side to move, 1 = of the other side, 2 = this decision is the last
+// stone of the turn.  Eight games per workgroup: their int8 boards are staged in LDS with
+// coalesced loads, then the 8 x 3 x cells output floats (a whole number of 16-byte units,
+// contiguous in memory) are written with 16-byte stores.
+// CELLS > 0 fixes the board size at compile time (divisions become multiplications).
+constexpr int kCanonGames = 8;
+template <int CELLS>
 __global__ __launch_bounds__(256) void canonical_input_kernel(const int8_t *__restrict__ boards,
                                                               const int8_t *__restrict__ player,
                                                               const int8_t *__restrict__ stones_left,
-                                                              long long total, int cells,
+                                                              long long num, int cells_arg,
                                                               float *__restrict__ out) {
-  const long long stride = (long long)gridDim.x * blockDim.x;
-  for (long long f = (long long)blockIdx.x * blockDim.x + threadIdx.x; f < total; f += stride) {
-    const long long b = f / cells;
-    const int cell = (int)(f - b * cells);
-    const int stone = boards[f], me = player[b];
-    float *o = out + b * 3 * cells + cell;
-    o[0] = stone == me ? 1.0f : 0.0f;
-    o[cells] = stone == -me ? 1.0f : 0.0f;
-    o[2 * cells] = stones_left[b] == 1 ? 1.0f : 0.0f;
+  const int cells = CELLS > 0 ? CELLS : cells_arg;
+  extern __shared__ int8_t s_board[];  // kCanonGames * cells
+  __shared__ int s_me[kCanonGames];
+  __shared__ float s_last[kCanonGames];
+  const long long g0 = (long long)blockIdx.x * kCanonGames;
+  const int ng = (int)(num - g0 < kCanonGames ? num - g0 : kCanonGames);
+  const int8_t *src = boards + g0 * cells;
+  for (int i = threadIdx.x; i < ng * cells; i += blockDim.x) s_board[i] = src[i];
+  if ((int)threadIdx.x < ng) {
+    s_me[threadIdx.x] = player[g0 + threadIdx.x];
+    s_last[threadIdx.x] = stones_left[g0 + threadIdx.x] == 1 ? 1.0f : 0.0f;
+  }
+  __syncthreads();
+  const int per_game = 3 * cells;
+  const int total = ng * per_game;
+  float *dst = out + g0 * per_game;
+  auto value = [&](int o) {
+    const int g = o / per_game, rem = o - g * per_game;
+    const int plane = rem / cells, cell = rem - plane * cells;
+    const int stone = s_board[g * cells + cell], me = s_me[g];
+    return plane == 2 ? s_last[g] : ((plane == 0 ? stone == me : stone == -me) ? 1.0f : 0.0f);
+  };
+  if ((total & 3) == 0 && (reinterpret_cast<uintptr_t>(dst) & 15u) == 0) {
+    for (int q = threadIdx.x; q < total / 4; q += blockDim.x) {
+      // two divisions per four outputs: locate the first, then step through planes and games
+      int g = (4 * q) / per_game, rem = 4 * q - g * per_game;
+      int plane = rem / cells, cell = rem - plane * cells;
+      f32x4 o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int stone = s_board[g * cells + cell], me = s_me[g];
+        o[e] = plane == 2 ? s_last[g] : ((plane == 0 ? stone == me : stone == -me) ? 1.0f : 0.0f);
+        if (++cell == cells) {
+          cell = 0;
+          if (++plane == 3) {
+            plane = 0;
+            g = g + 1 < ng ? g + 1 : g;
+          }
+        }
+      }
+      reinterpret_cast<f32x4 *>(dst)[q] = o;
+    }
+  } else {
+    for (int o = threadIdx.x; o < total; o += blockDim.x) dst[o] = value(o);
   }
 }
 
@@ -101,11 +140,14 @@ int launch_canonical_input(const int8_t *boards, const int8_t *player, const int
                            long long num, int n, float *out, hipStream_t st) {
   if (num == 0) return C6_OK;
   const int cells = n * n;
-  const long long total = num * cells;
-  long long blocks = (total + 255) / 256;
-  if (blocks > 256 * 64) blocks = 256 * 64;  // grid-stride beyond that
-  hipLaunchKernelGGL(canonical_input_kernel, dim3((unsigned)blocks), dim3(256), 0, st, boards, player,
-                     stones_left, total, cells, out);
+  const long long blocks = (num + kCanonGames - 1) / kCanonGames;
+  if (n == kBoard) {
+    hipLaunchKernelGGL(canonical_input_kernel<kPix>, dim3((unsigned)blocks), dim3(256),
+                       (size_t)kCanonGames * cells, st, boards, player, stones_left, num, cells, out);
+  } else {
+    hipLaunchKernelGGL(canonical_input_kernel<0>, dim3((unsigned)blocks), dim3(256),
+                       (size_t)kCanonGames * cells, st, boards, player, stones_left, num, cells, out);
+  }
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     set_error("canonical_input_kernel launch failed: %s", hipGetErrorString(e));

@@ -115,7 +115,8 @@ __global__ __launch_bounds__(256) void sample_kernel(const float *__restrict__ l
 }
 
 // out[p,plane,v] = x[plane, from_view(v,p)]   (connect6/train.py:222-230)
-// grid.y = view; each workgroup stages eight planes in LDS and writes the permuted planes.
+// Each workgroup stages eight planes in LDS once and writes all eight permuted views of them:
+// the input is read once, every output element is one LDS gather, stores are 16 bytes.
 constexpr int kExpandPlanes = 8;
 template <typename T>
 __global__ __launch_bounds__(256) void d4_expand_kernel(const T *__restrict__ x, long long planes,
@@ -125,34 +126,43 @@ __global__ __launch_bounds__(256) void d4_expand_kernel(const T *__restrict__ x,
   static_assert(SPAN % VEC == 0, "eight planes must be whole 16-byte units");
   typedef T vec_t __attribute__((ext_vector_type(VEC)));
   __shared__ __attribute__((aligned(16))) T s_in[SPAN];
-  __shared__ unsigned short s_map[kPix];
-  const int p = blockIdx.y;
   const long long plane0 = (long long)blockIdx.x * kExpandPlanes;
   const int np = (int)((planes - plane0) < kExpandPlanes ? (planes - plane0) : kExpandPlanes);
-  for (int v = threadIdx.x; v < kPix; v += blockDim.x) s_map[v] = (unsigned short)d4_from_view(v, p);
   const T *src = x + plane0 * kPix;
-  T *dst = out + ((size_t)p * planes + plane0) * kPix;
-  const bool aligned = ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u) == 0;
-  if (np == kExpandPlanes && aligned) {
+  T *dst0 = out + plane0 * kPix;                              // view p adds p * planes * kPix
+  const size_t view_stride = (size_t)planes * kPix;
+  const bool aligned = np == kExpandPlanes &&
+                       ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst0) |
+                         (view_stride * sizeof(T))) & 15u) == 0;
+  if (aligned) {
     for (int i = threadIdx.x; i < SPAN / VEC; i += blockDim.x)
       reinterpret_cast<vec_t *>(s_in)[i] = reinterpret_cast<const vec_t *>(src)[i];
-    __syncthreads();
+  } else {
+    for (int i = threadIdx.x; i < np * kPix; i += blockDim.x) s_in[i] = src[i];
+  }
+  __syncthreads();
+  if (aligned) {
     for (int i = threadIdx.x; i < SPAN / VEC; i += blockDim.x) {
-      vec_t o;
+      int pl[VEC], v[VEC];
 #pragma unroll
       for (int e = 0; e < VEC; ++e) {
         const int idx = i * VEC + e;
-        const int pl = idx / kPix, v = idx - pl * kPix;
-        o[e] = s_in[pl * kPix + s_map[v]];
+        pl[e] = idx / kPix;
+        v[e] = idx - pl[e] * kPix;
       }
-      reinterpret_cast<vec_t *>(dst)[i] = o;
+#pragma unroll
+      for (int p = 0; p < 8; ++p) {
+        vec_t o;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) o[e] = s_in[pl[e] * kPix + d4_from_view(v[e], p)];
+        reinterpret_cast<vec_t *>(dst0 + p * view_stride)[i] = o;
+      }
     }
   } else {
-    for (int i = threadIdx.x; i < np * kPix; i += blockDim.x) s_in[i] = src[i];
-    __syncthreads();
     for (int i = threadIdx.x; i < np * kPix; i += blockDim.x) {
       const int pl = i / kPix, v = i - pl * kPix;
-      dst[i] = s_in[pl * kPix + s_map[v]];
+#pragma unroll
+      for (int p = 0; p < 8; ++p) dst0[p * view_stride + i] = s_in[pl * kPix + d4_from_view(v, p)];
     }
   }
 }
@@ -267,7 +277,7 @@ int launch_sample(const float *logits, const uint8_t *legal, const float *u, flo
 
 int launch_d4_expand(const void *x, int elem_bytes, long long batch, void *out, hipStream_t st) {
   const long long planes = batch * 3;
-  const dim3 grid((unsigned)((planes + kExpandPlanes - 1) / kExpandPlanes), 8);
+  const dim3 grid((unsigned)((planes + kExpandPlanes - 1) / kExpandPlanes));
   if (elem_bytes == 4)
     hipLaunchKernelGGL(d4_expand_kernel<uint32_t>, grid, dim3(256), 0, st, (const uint32_t *)x,
                        planes, (uint32_t *)out);
