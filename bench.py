@@ -286,8 +286,15 @@ def main() -> int:
                 times.append(time.perf_counter() - t0)
         times.sort()
         med = times[len(times) // 2]
+        cpu_model = ""
+        try:
+            with open("/proc/cpuinfo") as fh:
+                cpu_model = next((ln.split(":", 1)[1].strip() for ln in fh if ln.startswith("model name")), "")
+        except OSError:
+            pass
         out["cpu_baseline"] = {
             "value": 256 / med, "unit": "boards/s", "cores": threads, "kind": "port",
+            "cpu_model": cpu_model, "os_cpu_count": os.cpu_count(),
             "sample": f"configs[0]: {len(times)} fp32 forwards of B=256 (same generator, same weights) "
                       f"with the PyTorch oracle, median",
         }
