@@ -61,6 +61,7 @@ struct PrecF32 {
   static constexpr int SPLIT = 0;
   static constexpr int LO8 = 0;
   static constexpr int LO6 = 0;
+  static constexpr int LO_FIRST = 1;  // first layer (0-based) whose input carries a low-order part
 };
 struct PrecBF16 {
   static constexpr int ID = C6_PREC_BF16;
@@ -68,6 +69,7 @@ struct PrecBF16 {
   static constexpr int SPLIT = 0;
   static constexpr int LO8 = 0;
   static constexpr int LO6 = 0;
+  static constexpr int LO_FIRST = 1;  // first layer (0-based) whose input carries a low-order part
 };
 struct PrecF16 {
   static constexpr int ID = C6_PREC_F16;
@@ -75,6 +77,7 @@ struct PrecF16 {
   static constexpr int SPLIT = 0;
   static constexpr int LO8 = 0;
   static constexpr int LO6 = 0;
+  static constexpr int LO_FIRST = 1;  // first layer (0-based) whose input carries a low-order part
 };
 struct PrecBF16X2 {
   static constexpr int ID = C6_PREC_BF16X2;
@@ -82,6 +85,7 @@ struct PrecBF16X2 {
   static constexpr int SPLIT = 1;     // activations stored as hi plane + lo plane, both bf16
   static constexpr int LO8 = 0;
   static constexpr int LO6 = 0;
+  static constexpr int LO_FIRST = 1;  // first layer (0-based) whose input carries a low-order part
 };
 struct PrecBF16F8 {
   static constexpr int ID = C6_PREC_BF16F8;
@@ -89,6 +93,7 @@ struct PrecBF16F8 {
   static constexpr int SPLIT = 0;
   static constexpr int LO8 = 1;       // bf16 plane + the dropped low-order part as scaled fp8
   static constexpr int LO6 = 0;
+  static constexpr int LO_FIRST = 1;  // first layer (0-based) whose input carries a low-order part
 };
 struct PrecBF16F6 {
   static constexpr int ID = C6_PREC_BF16F6;
@@ -96,6 +101,11 @@ struct PrecBF16F6 {
   static constexpr int SPLIT = 0;
   static constexpr int LO8 = 1;       // same record and fragment geometry as the fp8 mode ...
   static constexpr int LO6 = 1;       // ... with the low-order part as block-scaled fp6 (e2m3)
+  // Every 3x3 layer's input is corrected.  Correcting only the late layers is faster (+8 % from
+  // layer 5 on, +11 % from layer 6 on) but costs argmax agreement with fp32: over six weight seeds
+  // at B=4096 the mean / worst agreement is 99.23 / 99.10 % with all layers, 99.13 / 99.00 % from
+  // layer 4 on, 98.97 / 98.85 % from layer 5 on, 98.85 / 98.58 % from layer 6 on.
+  static constexpr int LO_FIRST = 1;
 };
 
 // bf16 + fp8 mode: what rounding an activation to bf16 drops (|lo| <= 2^-9 |a|) is kept as

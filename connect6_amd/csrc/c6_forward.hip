@@ -569,14 +569,15 @@ __device__ __forceinline__ void init_acc(f32x16 (&acc)[N][3], const float *__res
 }
 
 // barrier; every wave writes its share of the layer's output over the layer's input; barrier
-template <class P, int NT, class Pre>
+// (WITH_LO: the next layer runs a low-order pass, so its input needs the low-order part)
+template <class P, int NT, bool WITH_LO, class Pre>
 __device__ __forceinline__ void finish_layer(unsigned char *smem, const int (&ci)[3], int h,
                                              const f32x16 (&acc)[NT][3], Pre before_store) {
   __syncthreads();  // every wave has finished reading the layer's input
   before_store();
 #pragma unroll
   for (int j = 0; j < 3; ++j) {
-    if constexpr (P::LO6) {
+    if constexpr (P::LO6 && WITH_LO) {
       store_tile_lo6<P, NT>(smem, ci[j], h, acc, j);
     } else {
       store_tile<P, NT>(smem, ci[j], h, acc, j);
@@ -597,14 +598,16 @@ __device__ __forceinline__ void mid_layer(
   v4i lor0[LoRing<P, L>::D][LoRing<P, L>::NT], lor1[LoRing<P, L>::D][LoRing<P, L>::NT];
   conv3_pass<P, CIN, COUT>(smem, layer_weights<P, L>(packed, lane), ring, ci, h, acc);
   C6_MARK(30 + L);
-  if constexpr (P::LO8) lo_preload<P, L>(lor0, lor1, packed, lane);
-  if constexpr (P::LO8) conv3_lo_pass<P, L>(smem, packed, tail, lor0, lor1, ci, h, lane, acc);
+  if constexpr (P::LO8 && L >= P::LO_FIRST) {
+    lo_preload<P, L>(lor0, lor1, packed, lane);
+    conv3_lo_pass<P, L>(smem, packed, tail, lor0, lor1, ci, h, lane, acc);
+  }
   // With equal channel counts the main pass's over-read has already left the next layer's first
   // kRing k-steps in the ring (same fragment order, contiguous in memory): `next` is `ring`.
   if constexpr (kCoutArr[L + 1] != kCoutArr[L])
     preload_ring<kRing, kCoutArr[L + 1] / 32>(next, layer_weights<P, L + 1>(packed, lane));
   C6_MARK(4 + 2 * L);
-  finish_layer<P, NT>(smem, ci, h, acc, [] {});
+  finish_layer<P, NT, (L + 1 >= P::LO_FIRST)>(smem, ci, h, acc, [] {});
   C6_MARK(5 + 2 * L);
   (void)wave;
   (void)trace_on;
@@ -758,7 +761,7 @@ __global__ __launch_bounds__(256) void fused_forward_kernel(const FwdParams prm)
       conv1_pass<P>(smem, layer_weights<P, 0>(packed, lane), r1, l1base, acc);
       preload_ring<kRing, 1>(r2, layer_weights<P, 1>(packed, lane));
       C6_MARK(2);
-      finish_layer<P, 1>(smem, ci, h, acc, [&] {
+      finish_layer<P, 1, (1 >= P::LO_FIRST)>(smem, ci, h, acc, [&] {
         // the copies overlapped the activation tile: restore its zero padding
         for (int i = tidv; i < 60 * (G::PIXB / 16); i += THREADS) {
           const int k = i / (G::PIXB / 16), w16 = i - k * (G::PIXB / 16);
