@@ -261,3 +261,12 @@ def test_vector_env_refuses_cpu_device():
     with pytest.raises(RuntimeError, match="HIP device"):
         c6.canonical_network_input(torch.zeros(1, 9, 9, dtype=torch.int8), torch.ones(1, dtype=torch.int8),
                                    torch.ones(1, dtype=torch.int8))
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+
+    proc = subprocess.run([sys.executable, str(ROOT / "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert proc.returncode != 0
+    assert "one GPU" in proc.stderr and proc.stdout.strip() == ""
