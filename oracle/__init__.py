@@ -13,6 +13,8 @@ Contents
                 network in plain C (no library routine), used to pin
                 ``torch_ref`` on small inputs.
 ``cref``        ctypes binding of ``conv_ref.c``.
+``env_ref``     restatement of the batched environment step (``VectorConnect6.step``
+                with its local win check) plus an independent scalar game that pins it.
 
-Pinning status of every oracle function is listed in ``torch_ref``'s header.
+Pinning status of every oracle function is listed in the headers of ``torch_ref`` and ``env_ref``.
 """
