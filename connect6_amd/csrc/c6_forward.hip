@@ -144,13 +144,20 @@ __device__ __forceinline__ void put4(unsigned char *smem, int pbase, int sw, int
   }
 }
 
+// The 16-bit modes carry every pre-activation and activation multiplied by kActScale = -log2(e):
+// the packed first-layer weights and all biases are scaled by it, the head weights by its
+// inverse, and the weights of layers 2-8 not at all (their inputs already carry the factor).
+// SiLU then needs no multiply in front of its exp2:  u = kActScale * v  ->
+// u / (1 + 2^u) = kActScale * v * sigmoid(v).
+constexpr float kActScale = -1.4426950408889634f;
 template <class P> __device__ __forceinline__ float silu(float v) {
   if constexpr (P::EB == 4) {
     return v / (1.0f + expf(-v));
   } else {
-    return v * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(v * -1.4426950408889634f));
+    return v * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(v));
   }
 }
+template <class P> __host__ __device__ constexpr float act_scale() { return P::EB == 4 ? 1.0f : kActScale; }
 
 __device__ __forceinline__ float load_x(const void *x, int dt, size_t i) {
   if (dt == C6_DT_F32) return reinterpret_cast<const float *>(x)[i];
@@ -945,7 +952,7 @@ template <class P> __global__ void pack_kernel(const PackParams prm) {
       for (int e = 0; e < G::E; ++e) {
         const int kx = jj * G::E + e;
         float v = 0.0f;
-        if (row < kK1 * 3 && kx < kK1) v = w[((co * 3 + ch) * kK1 + ky) * kK1 + kx];
+        if (row < kK1 * 3 && kx < kK1) v = w[((co * 3 + ch) * kK1 + ky) * kK1 + kx] * act_scale<P>();
         put_elem<P>(dst, e, v);
       }
     } else {
@@ -966,11 +973,11 @@ template <class P> __global__ void pack_kernel(const PackParams prm) {
     if (ti < kBiasTotal) {
       int l = 0;
       while (ti >= bias_offset(l + 1)) ++l;
-      v = prm.conv_b[l] ? prm.conv_b[l][ti - bias_offset(l)] : 0.0f;
+      v = prm.conv_b[l] ? prm.conv_b[l][ti - bias_offset(l)] * act_scale<P>() : 0.0f;
     } else if (ti < kBiasTotal + kHeadC) {
-      v = prm.pol_w[ti - kBiasTotal];
+      v = prm.pol_w[ti - kBiasTotal] / act_scale<P>();
     } else if (ti < kBiasTotal + 2 * kHeadC) {
-      v = prm.val_w ? prm.val_w[ti - kBiasTotal - kHeadC] : 0.0f;
+      v = prm.val_w ? prm.val_w[ti - kBiasTotal - kHeadC] / act_scale<P>() : 0.0f;
     } else if (ti == kBiasTotal + 2 * kHeadC) {
       v = prm.pol_b ? prm.pol_b[0] : 0.0f;
     } else if (ti == kBiasTotal + 2 * kHeadC + 1) {

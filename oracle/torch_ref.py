@@ -134,22 +134,29 @@ def _bf16_round(t: torch.Tensor) -> torch.Tensor:
 
 
 def forward_bf16_emulated(
-    state: Mapping[str, torch.Tensor], x: torch.Tensor
+    state: Mapping[str, torch.Tensor], x: torch.Tensor, act_scale: float = 1.0
 ) -> tuple[torch.Tensor, torch.Tensor]:
-    """The arithmetic contract of the bf16 HIP path, emulated in fp32 torch:
+    """The arithmetic contract of the bf16 HIP paths, emulated in fp32 torch:
     conv weights and layer inputs rounded to bf16 (RNE), fp32 accumulation,
     bias + SiLU in fp32, ONE rounding to bf16 at each layer boundary, last
-    layer's activations and the two heads kept in fp32."""
+    layer's activations and the two heads kept in fp32.
+
+    ``act_scale`` c != 1 models the fused kernel, which carries c * activation
+    between layers (c = -log2 e): first-layer weights are rounded AFTER the
+    scaling, later layers see bf16(c * silu), biases are c * b in fp32, and the
+    heads divide the factor out again.  Mathematically the same network."""
     n = _num_layers(state)
+    c = float(act_scale)
     f = _bf16_round(x)
     for i in range(n):
         w = state[f"convs.{i}.weight"]
-        f = F.conv2d(f, _bf16_round(w), state[f"convs.{i}.bias"], stride=1, padding=w.shape[-1] // 2)
-        f = F.silu(f)
+        wq = _bf16_round(w * c) if i == 0 else _bf16_round(w)
+        u = F.conv2d(f, wq, state[f"convs.{i}.bias"] * c, stride=1, padding=w.shape[-1] // 2)
+        f = c * F.silu(u / c)
         if i + 1 < n:
             f = _bf16_round(f)
-    logits = F.conv2d(f, state["policy_output.weight"], state["policy_output.bias"]).flatten(1)
-    vmap = F.conv2d(f, state["value_output.weight"], state["value_output.bias"])
+    logits = F.conv2d(f, state["policy_output.weight"] / c, state["policy_output.bias"]).flatten(1)
+    vmap = F.conv2d(f, state["value_output.weight"] / c, state["value_output.bias"])
     value = torch.tanh(vmap.mean(dim=(-2, -1))).squeeze(1)
     return logits, value
 
