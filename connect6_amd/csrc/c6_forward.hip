@@ -79,8 +79,24 @@ template <class P> __device__ __forceinline__ int pack2(float a, float b) {
     return __builtin_bit_cast(int, __builtin_convertvector(v, bf16x2));
   }
 }
-__device__ __forceinline__ float bf16_lo(int w) { return __builtin_bit_cast(float, w << 16); }
-__device__ __forceinline__ float bf16_hi(int w) { return __builtin_bit_cast(float, w & (int)0xffff0000); }
+// What rounding to bf16 dropped: a - float(low half of w) and b - float(high half of w), each
+// ONE v_dot2c_f32_bf16 (acc + w.lo * m.lo + w.hi * m.hi with m = {-1, 0} or {0, -1}) instead of
+// an unpack and a subtract.  The difference is exactly representable, so the result is exact.
+// The multiplier pairs must sit in registers: as inline constants the compiler encodes them wrongly.
+struct DropConsts {
+  bf16x2 lo, hi;
+};
+template <class P> __device__ __forceinline__ DropConsts drop_consts() {
+  unsigned b0 = 0x0000BF80u, b1 = 0xBF800000u;
+  if constexpr (P::LO8) asm volatile("" : "+v"(b0), "+v"(b1));  // (only the modes that use them)
+  return DropConsts{__builtin_bit_cast(bf16x2, b0), __builtin_bit_cast(bf16x2, b1)};
+}
+__device__ __forceinline__ float dropped_lo(float a, int w, const DropConsts &k) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, w), k.lo, a, false);
+}
+__device__ __forceinline__ float dropped_hi(float b, int w, const DropConsts &k) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, w), k.hi, b, false);
+}
 
 // XOR term of the granule swizzle for position `pos` (0 for the padded layout)
 template <class P> __device__ __forceinline__ int swz_of(int pos) {
@@ -100,7 +116,7 @@ template <> struct Packed4<PrecF32> {
   f32x4 v;
 };
 
-template <class P> __device__ __forceinline__ Packed4<P> pack4(const float (&v)[4]) {
+template <class P> __device__ __forceinline__ Packed4<P> pack4(const float (&v)[4], const DropConsts &k) {
   Packed4<P> r;
   if constexpr (P::EB == 4) {
     r.v = f32x4{v[0], v[1], v[2], v[3]};
@@ -108,18 +124,21 @@ template <class P> __device__ __forceinline__ Packed4<P> pack4(const float (&v)[
     r.hi[0] = pack2<P>(v[0], v[1]);
     r.hi[1] = pack2<P>(v[2], v[3]);
     if constexpr (P::SPLIT) {
-      r.lo[0] = pack2<P>(v[0] - bf16_lo(r.hi[0]), v[1] - bf16_hi(r.hi[0]));
-      r.lo[1] = pack2<P>(v[2] - bf16_lo(r.hi[1]), v[3] - bf16_hi(r.hi[1]));
+      // (unpack and subtract here: the dot2 form measured 1.7 % slower in this mode)
+      r.lo[0] = pack2<P>(v[0] - __builtin_bit_cast(float, r.hi[0] << 16),
+                         v[1] - __builtin_bit_cast(float, r.hi[0] & (int)0xffff0000));
+      r.lo[1] = pack2<P>(v[2] - __builtin_bit_cast(float, r.hi[1] << 16),
+                         v[3] - __builtin_bit_cast(float, r.hi[1] & (int)0xffff0000));
     }
     if constexpr (P::LO8 && !P::LO6) {  // dropped low-order parts as four e4m3 bytes of lo * 2^kLoScaleLog2
       // v_cvt_scalef32_pk_fp8_f32 divides by its scale operand and turns overflow into NaN,
       // so the inputs are clamped to what 448 * 2^-kLoScaleLog2 can represent.
       constexpr float INV = 1.0f / (float)(1 << kLoScaleLog2), LIM = 448.0f * INV;
       typedef short v2s __attribute__((ext_vector_type(2)));
-      const float l0 = __builtin_amdgcn_fmed3f(v[0] - bf16_lo(r.hi[0]), -LIM, LIM);
-      const float l1 = __builtin_amdgcn_fmed3f(v[1] - bf16_hi(r.hi[0]), -LIM, LIM);
-      const float l2 = __builtin_amdgcn_fmed3f(v[2] - bf16_lo(r.hi[1]), -LIM, LIM);
-      const float l3 = __builtin_amdgcn_fmed3f(v[3] - bf16_hi(r.hi[1]), -LIM, LIM);
+      const float l0 = __builtin_amdgcn_fmed3f(dropped_lo(v[0], r.hi[0], k), -LIM, LIM);
+      const float l1 = __builtin_amdgcn_fmed3f(dropped_hi(v[1], r.hi[0], k), -LIM, LIM);
+      const float l2 = __builtin_amdgcn_fmed3f(dropped_lo(v[2], r.hi[1], k), -LIM, LIM);
+      const float l3 = __builtin_amdgcn_fmed3f(dropped_hi(v[3], r.hi[1], k), -LIM, LIM);
       v2s w = {0, 0};
       w = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(w, l0, l1, INV, false);
       w = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(w, l2, l3, INV, true);
@@ -455,11 +474,12 @@ __device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
 
 // SiLU of the four accumulators (tile t, pixel tile j, quad q): bias was added at init
 template <class P, int NT>
-__device__ __forceinline__ Packed4<P> silu_quad(const f32x16 (&acc)[NT][3], int t, int j, int q) {
+__device__ __forceinline__ Packed4<P> silu_quad(const f32x16 (&acc)[NT][3], int t, int j, int q,
+                                                 const DropConsts &k) {
   float v[4];
 #pragma unroll
   for (int e = 0; e < 4; ++e) v[e] = silu<P>(acc[t][j][4 * q + e]);
-  return pack4<P>(v);
+  return pack4<P>(v, k);
 }
 
 // SiLU + store of one pixel tile's accumulators (all cout tiles).  Lanes beyond pixel
@@ -474,11 +494,12 @@ __device__ __forceinline__ void store_tile(unsigned char *smem, int pos_in, int 
   asm volatile("" : "+v"(pos));
   const int pbase = pos * G::PIXB;
   const int sw = swz_of<P>(pos);
+  const DropConsts k = drop_consts<P>();
 #pragma unroll
   for (int t = 0; t < NT; ++t)
 #pragma unroll
     for (int q = 0; q < 4; ++q)
-      put4<P>(smem, pbase, sw, (32 * t + 8 * q + 4 * h) * G::EB, silu_quad<P, NT>(acc, t, j, q));
+      put4<P>(smem, pbase, sw, (32 * t + 8 * q + 4 * h) * G::EB, silu_quad<P, NT>(acc, t, j, q, k));
 }
 
 // fp6 mode: 32 low-order values of one position -> 24 bytes of e2m3 + the block's E8M0 scale.
@@ -521,6 +542,7 @@ __device__ __forceinline__ void store_tile_lo6(unsigned char *smem, int pos_in, 
   int pos = pos_in;
   asm volatile("" : "+v"(pos));
   unsigned char *rec = smem + pos * G::PIXB;
+  const DropConsts k = drop_consts<P>();
   float lo[NT][16];
 #pragma unroll
   for (int t = 0; t < NT; ++t)
@@ -531,10 +553,10 @@ __device__ __forceinline__ void store_tile_lo6(unsigned char *smem, int pos_in, 
       for (int e = 0; e < 4; ++e) v[e] = silu<P>(acc[t][j][4 * q + e]);
       const v2i hi = {pack2<P>(v[0], v[1]), pack2<P>(v[2], v[3])};
       *reinterpret_cast<v2i *>(rec + (32 * t + 8 * q + 4 * h) * 2) = hi;
-      lo[t][4 * q + 0] = v[0] - bf16_lo(hi[0]);
-      lo[t][4 * q + 1] = v[1] - bf16_hi(hi[0]);
-      lo[t][4 * q + 2] = v[2] - bf16_lo(hi[1]);
-      lo[t][4 * q + 3] = v[3] - bf16_hi(hi[1]);
+      lo[t][4 * q + 0] = dropped_lo(v[0], hi[0], k);
+      lo[t][4 * q + 1] = dropped_hi(v[1], hi[0], k);
+      lo[t][4 * q + 2] = dropped_lo(v[2], hi[1], k);
+      lo[t][4 * q + 3] = dropped_hi(v[3], hi[1], k);
     }
   if constexpr (NT >= 2) lo6_block(rec + G::LO_OFF + 32 * h, lo[0], lo[1], true);
   if constexpr (NT % 2 == 1) {
