@@ -303,3 +303,16 @@ def test_headline_mode_keeps_the_argmax_gate_on_other_weights(cuda, seed):
             agree = float((got.argmax(1) == want.argmax(1)).float().mean())
             print(f"seed {seed} {prec}: argmax agreement {agree:.4f}")
             assert agree >= ARGMAX_MIN
+
+
+def test_c_abi_from_a_plain_cpp_program(cuda):
+    # no Python between the caller and the library: dlopen, raw HIP pointers, brute-force C oracle
+    import subprocess
+    from pathlib import Path
+
+    exe = Path(__file__).resolve().parent / "c_abi" / "_build" / "c_abi_forward"
+    assert exe.exists(), "build it with __graft_entry__.build() (it is compiled there, not in the test)"
+    proc = subprocess.run([str(exe), str(_lib._SO)], capture_output=True, text=True, timeout=120)
+    print(proc.stdout)
+    assert proc.returncode == 0, proc.stdout + proc.stderr
+    assert "all checks passed" in proc.stdout
