@@ -1,27 +1,62 @@
 // Device helpers shared by the connect6_amd kernels (wave64 reductions, sampling, D4 maps).
 #pragma once
+#include <type_traits>
+
 #include "c6_common.h"
 
 namespace c6 {
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+// Wave64 all-reduce without LDS traffic: DPP inside a row of 16 lanes (quad swaps, then the
+// mirrored lane of the 8- and the 16-group, which belongs to the half not yet combined), then
+// v_permlane16_swap / v_permlane32_swap across rows.  Every lane ends with the result.
+template <class Op> __device__ __forceinline__ int wave_allreduce_bits(int v, Op op) {
+  v = op(v, __builtin_amdgcn_update_dpp(v, v, 0xB1, 0xF, 0xF, false));   // quad_perm [1,0,3,2]
+  v = op(v, __builtin_amdgcn_update_dpp(v, v, 0x4E, 0xF, 0xF, false));   // quad_perm [2,3,0,1]
+  v = op(v, __builtin_amdgcn_update_dpp(v, v, 0x141, 0xF, 0xF, false));  // row_half_mirror
+  v = op(v, __builtin_amdgcn_update_dpp(v, v, 0x140, 0xF, 0xF, false));  // row_mirror
+  {
+    const auto r = __builtin_amdgcn_permlane16_swap((unsigned)v, (unsigned)v, false, false);
+    const unsigned r0 = r[0], r1 = r[1];  // this row's and the neighbouring row's value
+    v = op((int)r0, (int)r1);
+  }
+  {
+    const auto r = __builtin_amdgcn_permlane32_swap((unsigned)v, (unsigned)v, false, false);
+    const unsigned r0 = r[0], r1 = r[1];  // this half's and the other half's value
+    v = op((int)r0, (int)r1);
+  }
   return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+  return __builtin_bit_cast(float, wave_allreduce_bits(__builtin_bit_cast(int, v), [](int a, int b) {
+    return __builtin_bit_cast(int, __builtin_bit_cast(float, a) + __builtin_bit_cast(float, b));
+  }));
 }
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-  return v;
+  return __builtin_bit_cast(float, wave_allreduce_bits(__builtin_bit_cast(int, v), [](int a, int b) {
+    return __builtin_bit_cast(int, fmaxf(__builtin_bit_cast(float, a), __builtin_bit_cast(float, b)));
+  }));
 }
 __device__ __forceinline__ int wave_min_i(int v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = min(v, __shfl_xor(v, o, 64));
-  return v;
+  return wave_allreduce_bits(v, [](int a, int b) { return a < b ? a : b; });
 }
 __device__ __forceinline__ int wave_max_i(int v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = max(v, __shfl_xor(v, o, 64));
+  return wave_allreduce_bits(v, [](int a, int b) { return a > b ? a : b; });
+}
+// Inclusive prefix sum over the 64 lanes: shifts inside each row of 16 (lanes without a source
+// add 0), then the totals of the rows before: lane 15 of rows 0 and 2 into rows 1 and 3, lane
+// 31 (by then the total of rows 0-1) into rows 2 and 3.
+__device__ __forceinline__ float wave_inclusive_sum(float v) {
+  auto shifted = [](float x, auto ctrl, auto rows) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), decltype(ctrl)::value,
+                                                                 decltype(rows)::value, 0xF, false));
+  };
+  using std::integral_constant;
+  v += shifted(v, integral_constant<int, 0x111>{}, integral_constant<int, 0xF>{});  // row_shr:1
+  v += shifted(v, integral_constant<int, 0x112>{}, integral_constant<int, 0xF>{});  // row_shr:2
+  v += shifted(v, integral_constant<int, 0x114>{}, integral_constant<int, 0xF>{});  // row_shr:4
+  v += shifted(v, integral_constant<int, 0x118>{}, integral_constant<int, 0xF>{});  // row_shr:8
+  v += shifted(v, integral_constant<int, 0x142>{}, integral_constant<int, 0xA>{});  // row_bcast:15 -> rows 1, 3
+  v += shifted(v, integral_constant<int, 0x143>{}, integral_constant<int, 0xC>{});  // row_bcast:31 -> rows 2, 3
   return v;
 }
 
@@ -55,13 +90,8 @@ __device__ __forceinline__ void wave_sample(int lane, float u, FZ z, FOK ok, int
     local += ex[e];
   }
   // inclusive scan of lane sums
-  float incl = local;
-#pragma unroll
-  for (int o = 1; o < 64; o <<= 1) {
-    const float t = __shfl_up(incl, o, 64);
-    if (lane >= o) incl += t;
-  }
-  const float total = __shfl(incl, 63, 64);
+  const float incl = wave_inclusive_sum(local);
+  const float total = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, incl), 63));
   const float target = u * total;
   float run = incl - local;
   int first = 1 << 30;

@@ -849,7 +849,12 @@ __global__ __launch_bounds__(256) void fused_forward_kernel(const FwdParams prm)
       const float polb = valw[kHeadC], valb = valw[kHeadC + 1];
       float tot[3];
 #pragma unroll
-      for (int j = 0; j < 3; ++j) tot[j] = pol[j] + __shfl_xor(pol[j], 32, 64);
+      for (int j = 0; j < 3; ++j) {  // add the other lane half's channels
+        const unsigned bits = __builtin_bit_cast(unsigned, pol[j]);
+        const auto r = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+        const unsigned r0 = r[0], r1 = r[1];
+        tot[j] = __builtin_bit_cast(float, r0) + __builtin_bit_cast(float, r1);
+      }
 #pragma unroll
       for (int j = 0; j < 3; ++j)
         if (h == 0 && valid[j]) lgt[pix[j]] = tot[j] + polb;
