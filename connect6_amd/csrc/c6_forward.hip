@@ -200,17 +200,42 @@ template <class P> struct L1Pipe {
 };
 
 // fragments (k-step s, cout tile t) of a layer with NT cout tiles sit at index s*NT + t
+// A run of 1 KiB weight fragments of one packed buffer, read 16 bytes per lane with buffer loads:
+// the fragment's offset travels in a scalar register and the lane's part (lane * 16) in one
+// vector register that never changes, so a load needs no per-lane 64-bit address arithmetic and
+// issues in a few cycles (a global load with a per-lane address costs the wave ~20-30 cycles of
+// issue time next to MFMAs; measured, this form ~2).
+struct WFrags {
+  __amdgpu_buffer_rsrc_t rsrc;
+  int lane_off;  // lane * 16
+  int base;      // byte offset of fragment 0 (wave-uniform)
+  __device__ __forceinline__ v4i operator[](int f) const {
+    return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_off, base + f * 1024, 0));
+  }
+  __device__ __forceinline__ v2i first8(int f) const {  // the first 8 of the lane's 16 bytes
+    return __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(rsrc, lane_off, base + f * 1024, 0));
+  }
+  __device__ __forceinline__ WFrags operator+(int f) const { return WFrags{rsrc, lane_off, base + f * 1024}; }
+};
+template <class P>
+__device__ __forceinline__ WFrags packed_frags(const unsigned char *packed, int lane, int frag) {
+  // (packed is the same for every lane: a board's weight set)
+  return WFrags{__builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char *>(packed), 0,
+                                                  (int)Geo<P>::TAIL_OFF, 0x00020000),
+                lane * 16, frag * 1024};
+}
+
 template <int D, int NT>
-__device__ __forceinline__ void preload_ring(v4i (&ring)[D][NT], const v4i *__restrict__ wl) {
+__device__ __forceinline__ void preload_ring(v4i (&ring)[D][NT], const WFrags &wl) {
 #pragma unroll
   for (int d = 0; d < D; ++d)
 #pragma unroll
-    for (int t = 0; t < NT; ++t) ring[d][t] = wl[(d * NT + t) * 64];
+    for (int t = 0; t < NT; ++t) ring[d][t] = wl[d * NT + t];
 }
 
 template <class P, int L>
-__device__ __forceinline__ const v4i *layer_weights(const unsigned char *packed, int lane) {
-  return reinterpret_cast<const v4i *>(packed + (size_t)Geo<P>::frag_offset(L) * 1024) + lane;
+__device__ __forceinline__ WFrags layer_weights(const unsigned char *packed, int lane) {
+  return packed_frags<P>(packed, lane, Geo<P>::frag_offset(L));
 }
 
 constexpr int kAhead = 2;  // k-steps between the LDS read of an activation fragment and its MFMAs
@@ -233,7 +258,7 @@ template <int N_MFMA, int N_DSREAD, int N_VMEM> __device__ __forceinline__ void 
 // first layer: 23x23 on 3 planes, K = (ky, plane, kx24) split over lane halves
 // ------------------------------------------------------------------------
 template <class P>
-__device__ __forceinline__ void conv1_pass(const unsigned char *smem, const v4i *__restrict__ wl,
+__device__ __forceinline__ void conv1_pass(const unsigned char *smem, const WFrags &wl,
                                            v4i (&ring)[L1Pipe<P>::D][1], const int (&l1base)[3],
                                            f32x16 (&acc)[1][3]) {
   using G = Geo<P>;
@@ -253,7 +278,7 @@ __device__ __forceinline__ void conv1_pass(const unsigned char *smem, const v4i 
 #pragma unroll 1
   for (int it = 0; it < ITERS; ++it) {
     const int adv = it * PP::ROWS_BODY * ROWB;
-    const v4i *wn = wl + (size_t)(it * U + D) * 64;
+    const WFrags wn = wl + (it * U + D);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       // after the last steps this reads the zero row / the next copy, which is harmless
@@ -264,7 +289,7 @@ __device__ __forceinline__ void conv1_pass(const unsigned char *smem, const v4i 
         bq[un % (kAhead + 1)][j] = *reinterpret_cast<const v4i *>(smem + l1base[j] + adv + offn);
 #pragma unroll
       for (int j = 0; j < 3; ++j) mma<P>(ring[u % D][0], bq[u % (kAhead + 1)][j], acc[0][j]);
-      ring[u % D][0] = wn[u * 64];  // k-step it*U + u + D (the tail over-reads the next layer)
+      ring[u % D][0] = wn[u];  // k-step it*U + u + D (the tail over-reads the next layer)
       interleave_step<3 * (P::EB == 4 ? 4 : 1), 3, 1>();
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -275,7 +300,7 @@ __device__ __forceinline__ void conv1_pass(const unsigned char *smem, const v4i 
 // 3x3 layers: K = (tap, cin), cin fastest; taps are constant position offsets
 // ------------------------------------------------------------------------
 template <class P, int CIN, int COUT>
-__device__ __forceinline__ void conv3_pass(const unsigned char *smem, const v4i *__restrict__ wl,
+__device__ __forceinline__ void conv3_pass(const unsigned char *smem, const WFrags &wl,
                                            v4i (&ring)[kRing][COUT / 32], const int (&ci)[3], int h,
                                            f32x16 (&acc)[COUT / 32][3]) {
   using G = Geo<P>;
@@ -317,7 +342,7 @@ __device__ __forceinline__ void conv3_pass(const unsigned char *smem, const v4i 
 
 #pragma unroll 1
   for (int ky = 0; ky < 3; ++ky) {
-    const v4i *wn = wl + (size_t)(ky * U + D) * NT * 64;
+    const WFrags wn = wl + (ky * U + D) * NT;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       // fetch the activation fragments of k-step u + kAhead while this step's MFMAs run
@@ -343,7 +368,7 @@ __device__ __forceinline__ void conv3_pass(const unsigned char *smem, const v4i 
       }
       // weights of k-step u+D (the tail over-reads into the next layer)
 #pragma unroll
-      for (int t = 0; t < NT; ++t) ring[u % D][t] = wn[(u * NT + t) * 64];
+      for (int t = 0; t < NT; ++t) ring[u % D][t] = wn[u * NT + t];
       interleave_step<NT * 3 * (P::SPLIT ? 2 : 1) * (P::EB == 4 ? 4 : 1), 3 * (P::SPLIT ? 2 : 1), NT>();
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -359,32 +384,32 @@ __device__ __forceinline__ void conv3_pass(const unsigned char *smem, const v4i 
 // piece 1 = 16 or 8.  (Filling the ring before the layer's main pass was measured slower: the
 // extra loads and registers cost the main pass more than the second pass gains.)
 template <class P>
-__device__ __forceinline__ void lo_load_pieces(const v4i *src, v4i &p0, v4i &p1) {
+__device__ __forceinline__ void lo_load_pieces(const WFrags &src, v4i &p0, v4i &p1) {
   p0 = src[0];
   if constexpr (P::LO6) {
-    const v2i q = *reinterpret_cast<const v2i *>(src + 64);
+    const v2i q = src.first8(1);
     p1 = v4i{q[0], q[1], 0, 0};
   } else {
-    p1 = src[64];
+    p1 = src[1];
   }
 }
 template <class P, int L> struct LoRing {
   static constexpr int NT = kCoutArr[L] / 32;
   static constexpr int NC = Geo<P>::lo_chunks(L);
   static constexpr int D = P::LO8 ? (NC < kLoRing ? NC : kLoRing) : 1;  // ring depth in 64-wide chunks
-  __device__ __forceinline__ static const v4i *base(const unsigned char *packed, int lane) {
-    return reinterpret_cast<const v4i *>(packed + (size_t)Geo<P>::lo_frag_offset(L) * 1024) + lane;
+  __device__ __forceinline__ static WFrags base(const unsigned char *packed, int lane) {
+    return packed_frags<P>(packed, lane, Geo<P>::lo_frag_offset(L));
   }
 };
 template <class P, int L, int D, int NT>
 __device__ __forceinline__ void lo_preload(v4i (&f0)[D][NT], v4i (&f1)[D][NT],
                                            const unsigned char *packed, int lane) {
   static_assert(D == LoRing<P, L>::D && NT == LoRing<P, L>::NT, "ring shape");
-  const v4i *wl = LoRing<P, L>::base(packed, lane);
+  const WFrags wl = LoRing<P, L>::base(packed, lane);
 #pragma unroll
   for (int d = 0; d < D; ++d)
 #pragma unroll
-    for (int t = 0; t < NT; ++t) lo_load_pieces<P>(wl + (d * NT + t) * 2 * 64, f0[d][t], f1[d][t]);
+    for (int t = 0; t < NT; ++t) lo_load_pieces<P>(wl + (d * NT + t) * 2, f0[d][t], f1[d][t]);
   __builtin_amdgcn_sched_barrier(0);  // issue here: do not sink the loads to their first use
 }
 
@@ -401,7 +426,7 @@ __device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
   constexpr int PER32 = kCinArr[L] / 32;
   constexpr int HC = G::lo_half_chunks(L), NC = G::lo_chunks(L);
   typedef int v8i __attribute__((ext_vector_type(8)));
-  const v4i *wl = LoRing<P, L>::base(packed, lane);
+  const WFrags wl = LoRing<P, L>::base(packed, lane);
   const int sw = reinterpret_cast<const int *>(tail)[G::TAIL_SW + L];
   const int scale_w = 127 - sw;            // E8M0 exponent undoing the weight copy's 2^sw
   const int scale_x = 127 - kLoScaleLog2;  // ... and the activations' 2^kLoScaleLog2 (fp8 mode)
@@ -441,7 +466,7 @@ __device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
   for (int a = 0; a < kAhead; ++a) fetch(a, bq[a]);
 #pragma unroll 1
   for (int c0 = 0; c0 < NC; c0 += D) {
-    const v4i *wn = wl + (size_t)(c0 + D) * NT * 2 * 64;
+    const WFrags wn = wl + (c0 + D) * NT * 2;
 #pragma unroll
     for (int d = 0; d < D; ++d) {
       if (NC % D != 0 && d >= NC % D && c0 + d >= NC) continue;  // the last group may be short
@@ -465,7 +490,7 @@ __device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
       }
       // weights of chunk c0 + d + D (the tail over-reads the next layer's copy or the zero padding)
 #pragma unroll
-      for (int t = 0; t < NT; ++t) lo_load_pieces<P>(wn + (d * NT + t) * 2 * 64, ring0[d][t], ring1[d][t]);
+      for (int t = 0; t < NT; ++t) lo_load_pieces<P>(wn + (d * NT + t) * 2, ring0[d][t], ring1[d][t]);
       interleave_step<NT * 3, 2 * 3, 2 * NT>();
       __builtin_amdgcn_sched_barrier(0);
     }
