@@ -199,7 +199,6 @@ template <class P> struct L1Pipe {
   static_assert(U % D == 0 && ITERS * ROWS_BODY == kL1RowsHalf, "first-layer pipeline shape");
 };
 
-// fragments (k-step s, cout tile t) of a layer with NT cout tiles sit at index s*NT + t
 // A run of 1 KiB weight fragments of one packed buffer, read 16 bytes per lane with buffer loads:
 // the fragment's offset travels in a scalar register and the lane's part (lane * 16) in one
 // vector register that never changes, so a load needs no per-lane 64-bit address arithmetic and
@@ -225,6 +224,7 @@ __device__ __forceinline__ WFrags packed_frags(const unsigned char *packed, int 
                 lane * 16, frag * 1024};
 }
 
+// fragments (k-step s, cout tile t) of a layer with NT cout tiles sit at index s*NT + t
 template <int D, int NT>
 __device__ __forceinline__ void preload_ring(v4i (&ring)[D][NT], const WFrags &wl) {
 #pragma unroll
