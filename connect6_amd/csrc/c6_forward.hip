@@ -417,7 +417,7 @@ __device__ __forceinline__ void lo_preload(v4i (&f0)[D][NT], v4i (&f1)[D][NT],
 // every fragment load of the layer to the front.
 template <class P, int L, int D, int NT>
 __device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
-                                              const unsigned char *packed, const float *tail,
+                                              const unsigned char *packed, int scale_w,
                                               v4i (&ring0)[D][NT], v4i (&ring1)[D][NT],
                                               const int (&ci)[3], int h, int lane,
                                               f32x16 (&acc)[NT][3]) {
@@ -427,8 +427,9 @@ __device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
   constexpr int HC = G::lo_half_chunks(L), NC = G::lo_chunks(L);
   typedef int v8i __attribute__((ext_vector_type(8)));
   const WFrags wl = LoRing<P, L>::base(packed, lane);
-  const int sw = reinterpret_cast<const int *>(tail)[G::TAIL_SW + L];
-  const int scale_w = 127 - sw;            // E8M0 exponent undoing the weight copy's 2^sw
+  // scale_w: E8M0 exponent undoing the weight copy's 2^sw.  (It arrives as an argument, read once
+  // per board: a load here would be the newest of ~36 loads in flight, and waiting for it before the
+  // first MFMA would drain them all.)
   const int scale_x = 127 - kLoScaleLog2;  // ... and the activations' 2^kLoScaleLog2 (fp8 mode)
   (void)scale_x;
 
@@ -646,7 +647,7 @@ template <class P, int L>
 __device__ __forceinline__ void mid_layer(
     unsigned char *smem, const unsigned char *packed, const float *tail,
     v4i (&ring)[kRing][kCoutArr[L] / 32], v4i (&next)[kRing][kCoutArr[L + 1] / 32],
-    const int (&ci)[3], int h, int lane, int wave, bool trace_on) {
+    const int (&ci)[3], int h, int lane, int wave, bool trace_on, const int (&lo_scale_w)[8]) {
   constexpr int CIN = kCinArr[L], COUT = kCoutArr[L], NT = COUT / 32;
   f32x16 acc[NT][3];
   init_acc(acc, tail + bias_offset(L), h);
@@ -655,7 +656,7 @@ __device__ __forceinline__ void mid_layer(
   C6_MARK(30 + L);
   if constexpr (P::LO8 && L >= P::LO_FIRST) {
     lo_preload<P, L>(lor0, lor1, packed, lane);
-    conv3_lo_pass<P, L>(smem, packed, tail, lor0, lor1, ci, h, lane, acc);
+    conv3_lo_pass<P, L>(smem, packed, lo_scale_w[L], lor0, lor1, ci, h, lane, acc);
   }
   // With equal channel counts the main pass's over-read has already left the next layer's first
   // kRing k-steps in the ring (same fragment order, contiguous in memory): `next` is `ring`.
@@ -765,6 +766,13 @@ __global__ __launch_bounds__(256) void fused_forward_kernel(const FwdParams prm)
     asm volatile("" : "+v"(tidv));
     const unsigned char *packed = packed_of(b);
     const float *tail = reinterpret_cast<const float *>(packed + G::TAIL_OFF);
+    // block-scale exponents of the low-order weight copies (E8M0: 127 - log2 of the copy's scale),
+    // fetched here, long before any second pass needs them
+    int lo_scale_w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if constexpr (P::LO8) {
+#pragma unroll
+      for (int l = 1; l < 8; ++l) lo_scale_w[l] = 127 - reinterpret_cast<const int *>(tail)[G::TAIL_SW + l];
+    }
 
 #ifdef C6_TRACE
     const bool trace_on = (b == b_first + 2);  // third board of this workgroup
@@ -828,12 +836,12 @@ __global__ __launch_bounds__(256) void fused_forward_kernel(const FwdParams prm)
       });
     }
     C6_MARK(3);
-    mid_layer<P, 1>(smem, packed, tail, r2, r345, ci, h, lane, wave, trace_on);
-    mid_layer<P, 2>(smem, packed, tail, r345, r345, ci, h, lane, wave, trace_on);
-    mid_layer<P, 3>(smem, packed, tail, r345, r345, ci, h, lane, wave, trace_on);
-    mid_layer<P, 4>(smem, packed, tail, r345, r678, ci, h, lane, wave, trace_on);
-    mid_layer<P, 5>(smem, packed, tail, r678, r678, ci, h, lane, wave, trace_on);
-    mid_layer<P, 6>(smem, packed, tail, r678, r678, ci, h, lane, wave, trace_on);
+    mid_layer<P, 1>(smem, packed, tail, r2, r345, ci, h, lane, wave, trace_on, lo_scale_w);
+    mid_layer<P, 2>(smem, packed, tail, r345, r345, ci, h, lane, wave, trace_on, lo_scale_w);
+    mid_layer<P, 3>(smem, packed, tail, r345, r345, ci, h, lane, wave, trace_on, lo_scale_w);
+    mid_layer<P, 4>(smem, packed, tail, r345, r678, ci, h, lane, wave, trace_on, lo_scale_w);
+    mid_layer<P, 5>(smem, packed, tail, r678, r678, ci, h, lane, wave, trace_on, lo_scale_w);
+    mid_layer<P, 6>(smem, packed, tail, r678, r678, ci, h, lane, wave, trace_on, lo_scale_w);
 
     // ---- layer 8 + both 1x1 heads straight from the fp32 accumulators ----
     {
@@ -848,7 +856,7 @@ __global__ __launch_bounds__(256) void fused_forward_kernel(const FwdParams prm)
       conv3_pass<P, 96, 96>(smem, layer_weights<P, 7>(packed, lane), r678, ci, h, acc);
       C6_MARK(37);
       if constexpr (P::LO8) lo_preload<P, 7>(lor0, lor1, packed, lane);
-      if constexpr (P::LO8) conv3_lo_pass<P, 7>(smem, packed, tail, lor0, lor1, ci, h, lane, acc);
+      if constexpr (P::LO8) conv3_lo_pass<P, 7>(smem, packed, lo_scale_w[7], lor0, lor1, ci, h, lane, acc);
       if (bn < b_end) preload_ring<L1Pipe<P>::D, 1>(r1, layer_weights<P, 0>(packed_of(bn), lane));
       C6_MARK(18);
       float pol[3] = {0.0f, 0.0f, 0.0f};
