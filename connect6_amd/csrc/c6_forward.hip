@@ -465,37 +465,44 @@ __device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
   v4i bq[kAhead + 1][3][2];
 #pragma unroll
   for (int a = 0; a < kAhead; ++a) fetch(a, bq[a]);
-#pragma unroll 1
-  for (int c0 = 0; c0 < NC; c0 += D) {
+  // chunk c0 + d: its MFMAs, the LDS reads of chunk c0 + d + kAhead and the refill of ring slot d
+  auto chunk = [&](int c0, int d) {
     const WFrags wn = wl + (c0 + D) * NT * 2;
+    v4i(&bcur)[3][2] = bq[d % (kAhead + 1)];
+    // (after the last chunks: harmless re-reads)
+    fetch(c0 + d + kAhead < NC ? c0 + d + kAhead : NC - 1, bq[(d + kAhead) % (kAhead + 1)]);
 #pragma unroll
-    for (int d = 0; d < D; ++d) {
-      if (NC % D != 0 && d >= NC % D && c0 + d >= NC) continue;  // the last group may be short
-      v4i(&bcur)[3][2] = bq[d % (kAhead + 1)];
-      // (after the last chunks: harmless re-reads)
-      fetch(c0 + d + kAhead < NC ? c0 + d + kAhead : NC - 1, bq[(d + kAhead) % (kAhead + 1)]);
+    for (int t = 0; t < NT; ++t) {
+      const v8i a = __builtin_shufflevector(ring0[d][t], ring1[d][t], 0, 1, 2, 3, 4, 5, 6, 7);
 #pragma unroll
-      for (int t = 0; t < NT; ++t) {
-        const v8i a = __builtin_shufflevector(ring0[d][t], ring1[d][t], 0, 1, 2, 3, 4, 5, 6, 7);
-#pragma unroll
-        for (int j = 0; j < 3; ++j) {
-          const v8i b = __builtin_shufflevector(bcur[j][0], bcur[j][1], 0, 1, 2, 3, 4, 5, 6, 7);
-          if constexpr (P::LO6) {
-            acc[t][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[t][j], 2, 2, 0,
-                                                                             scale_w, 0, b[6]);
-          } else {
-            acc[t][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[t][j], 0, 0, 0,
-                                                                             scale_w, 0, scale_x);
-          }
+      for (int j = 0; j < 3; ++j) {
+        const v8i b = __builtin_shufflevector(bcur[j][0], bcur[j][1], 0, 1, 2, 3, 4, 5, 6, 7);
+        if constexpr (P::LO6) {
+          acc[t][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[t][j], 2, 2, 0,
+                                                                           scale_w, 0, b[6]);
+        } else {
+          acc[t][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[t][j], 0, 0, 0,
+                                                                           scale_w, 0, scale_x);
         }
       }
-      // weights of chunk c0 + d + D (the tail over-reads the next layer's copy or the zero padding)
-#pragma unroll
-      for (int t = 0; t < NT; ++t) lo_load_pieces<P>(wn + (d * NT + t) * 2, ring0[d][t], ring1[d][t]);
-      interleave_step<NT * 3, 2 * 3, 2 * NT>();
-      __builtin_amdgcn_sched_barrier(0);
     }
+    // weights of chunk c0 + d + D (the tail over-reads the next layer's copy or the zero padding)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) lo_load_pieces<P>(wn + (d * NT + t) * 2, ring0[d][t], ring1[d][t]);
+    interleave_step<NT * 3, 2 * 3, 2 * NT>();
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // Whole groups of D chunks in a runtime loop with a single basic block (a branch inside the
+  // body makes the compiler wait for every LDS read in flight at each group boundary), then the
+  // NC % D chunks that are left, unrolled.
+  constexpr int WHOLE = NC / D * D;
+#pragma unroll 1
+  for (int c0 = 0; c0 < WHOLE; c0 += D) {
+#pragma unroll
+    for (int d = 0; d < D; ++d) chunk(c0, d);
   }
+#pragma unroll
+  for (int d = 0; d < NC % D; ++d) chunk(WHOLE, d);
 }
 
 // SiLU of the four accumulators (tile t, pixel tile j, quad q): bias was added at init
