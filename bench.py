@@ -92,7 +92,7 @@ def main() -> int:
     value = B / wall
     achieved = B * CONV_FLOP_PER_BOARD / kern / 1e12
     out = {
-        "metric": "boards/sec B=4096 16-bit forward (masked logits + value), 1x MI355X",
+        "metric": "boards/sec B=4096 bf16 forward + % MFMA peak; G=8 grouped-history boards/sec",
         "value": value,
         "unit": "boards/s",
         "n_gpus": 1,

@@ -5,7 +5,7 @@ Host-side mirror of the reference's operator interface for this path
 a C-ABI library of hand-written HIP kernels.
 """
 from ._lib import C6Error, build, load
-from .history import HistoricalCheckpoint, HistoricalPolicyEnsemble
+from .history import HistoricalCheckpoint, HistoricalPolicyEnsemble, history_dtype
 from .model import PolicyValueNet, build_model, mask_logits
 from .selfplay import (
     d4_expand,
@@ -33,6 +33,7 @@ __all__ = [
     "d4_expand",
     "d4_reduce",
     "evaluate_d4",
+    "history_dtype",
     "inverse_transform_actions",
     "load",
     "mask_logits",

@@ -15,6 +15,7 @@ _CSRC = _PKG / "csrc"
 _LIBDIR = _PKG / "lib"
 _SO = _LIBDIR / "libconnect6_amd.so"
 _SOURCES = ("c6_forward.hip", "c6_tail.hip", "c6_generic.hip", "c6_env.hip", "c6_api.hip")
+_RESOURCES = _LIBDIR / "resource_usage.txt"   # registers, scratch and LDS of every kernel, written by build()
 
 # arithmetic modes (include/connect6_amd.h)
 PREC_F32, PREC_BF16, PREC_F16, PREC_BF16X2, PREC_BF16F8, PREC_BF16F6 = 0, 1, 2, 3, 4, 5
@@ -55,15 +56,41 @@ def build(verbose: bool = False) -> Path:
         # packed-fp32 VALU forms are disabled for every kernel in this library
         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
         "-Wall", "-Wno-unused-function",
+        "-Rpass-analysis=kernel-resource-usage",
         "-o", str(_SO),
     ] + [str(_CSRC / s) for s in _SOURCES]
     proc = subprocess.run(cmd, capture_output=True, text=True)
+    remarks, other = [], []
+    for line in proc.stderr.splitlines():
+        (remarks if "-Rpass-analysis=kernel-resource-usage" in line else other).append(line)
+    # (a remark is followed by a source excerpt of two lines; drop those too)
+    other = [ln for ln in other if not ln.lstrip().startswith(("|", "^")) and "__global__" not in ln]
     if verbose or proc.returncode != 0:
         print(proc.stdout)
-        print(proc.stderr)
+        print("\n".join(other))
     if proc.returncode != 0:
-        raise C6Error(f"hipcc failed ({proc.returncode}):\n{proc.stderr[-4000:]}")
+        raise C6Error(f"hipcc failed ({proc.returncode}):\n" + "\n".join(other)[-4000:])
+    _RESOURCES.write_text("\n".join(r.split("remark:", 1)[1].rsplit("[", 1)[0].rstrip() for r in remarks) + "\n")
     return _SO
+
+
+def resource_usage(rebuild_if_missing: bool = True) -> dict[str, dict[str, int]]:
+    """Per kernel (mangled name): registers, scratch bytes per lane, spills and LDS as the
+    compiler reported them in the last ``build()``."""
+    if not _RESOURCES.exists():
+        if not rebuild_if_missing:
+            raise C6Error(f"{_RESOURCES} is missing: run connect6_amd.build()")
+        build()
+    out: dict[str, dict[str, int]] = {}
+    cur = None
+    for line in _RESOURCES.read_text().splitlines():
+        key, _, val = line.strip().partition(":")
+        key = key.strip()
+        if key == "Function Name":
+            cur = out.setdefault(val.strip(), {})
+        elif cur is not None and val.strip().lstrip("-").isdigit():
+            cur[key.split(" [")[0]] = int(val)
+    return out
 
 
 _lib = None

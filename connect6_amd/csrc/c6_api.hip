@@ -1,4 +1,5 @@
 // extern "C" boundary of libconnect6_amd.so: argument validation and dispatch.
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -35,6 +36,41 @@ int launch_generic(const void *x, int x_dtype, long long batch, int n, int layer
 int launch_env_step(const EnvParams &p, hipStream_t st);
 int launch_canonical_input(const int8_t *boards, const int8_t *player, const int8_t *stones_left,
                            long long num, int n, float *out, hipStream_t st);
+
+// The kernels exist for gfx950 only.  Checked once per device, just before an entry point's
+// first launch there, so that another GPU gets C6_EARCH instead of a launch failure.
+static int device_ok(const char *who) {
+  constexpr int kMaxDevices = 64;
+  static std::atomic<int> state[kMaxDevices];  // 0 unknown, 1 gfx950, -1 something else
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    set_error("%s: no usable current device (%s)", who, hipGetErrorString(e));
+    return C6_ELAUNCH;
+  }
+  int s = state[dev].load(std::memory_order_relaxed);
+  if (s == 0) {
+    hipDeviceProp_t prop;
+    e = hipGetDeviceProperties(&prop, dev);
+    if (e != hipSuccess) {
+      set_error("%s: hipGetDeviceProperties failed: %s", who, hipGetErrorString(e));
+      return C6_ELAUNCH;
+    }
+    s = std::strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? 1 : -1;
+    if (s < 0) set_error("%s: device %d is %s; this library is built for gfx950 only", who, dev, prop.gcnArchName);
+    state[dev].store(s, std::memory_order_relaxed);
+  }
+  if (s < 0) {
+    set_error("%s: device %d is not gfx950; this library is built for gfx950 only", who, dev);
+    return C6_EARCH;
+  }
+  return C6_OK;
+}
+#define C6_REQUIRE_DEVICE(who)                  \
+  do {                                          \
+    const int rc_dev_ = device_ok(who);         \
+    if (rc_dev_ != C6_OK) return rc_dev_;       \
+  } while (0)
 
 static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 static int elem_bytes(int dt) { return dt == C6_DT_F32 ? 4 : ((dt == C6_DT_BF16 || dt == C6_DT_F16) ? 2 : 0); }
@@ -88,6 +124,7 @@ int c6_pack_weights(const float *const *conv_w, const float *const *conv_b, cons
   pp.val_w = val_w;
   pp.val_b = val_b;
   pp.packed = static_cast<unsigned char *>(packed);
+  C6_REQUIRE_DEVICE("c6_pack_weights");
   return dispatch_pack(prec, pp, static_cast<hipStream_t>(stream));
 }
 
@@ -153,6 +190,7 @@ int c6_forward(const void *x, int x_dtype, int64_t groups, int64_t boards_per_gr
   fp.index = nullptr;
   fp.num_states = 0;
   fp.view = 0;
+  C6_REQUIRE_DEVICE("c6_forward");
   return dispatch_forward(prec, fp, static_cast<hipStream_t>(stream));
 }
 
@@ -209,6 +247,7 @@ int c6_forward_boards(const int8_t *boards, const int8_t *player, const int8_t *
   fp.index = reinterpret_cast<const long long *>(index);
   fp.num_states = num_states;
   fp.view = view;
+  C6_REQUIRE_DEVICE("c6_forward_boards");
   return dispatch_forward(prec, fp, static_cast<hipStream_t>(stream));
 }
 
@@ -273,6 +312,7 @@ int c6_forward_generic(const void *x, int x_dtype, int64_t batch, int board, int
     set_error("c6_forward_generic: bad mask_mode %d", mask_mode);
     return C6_EINVAL;
   }
+  C6_REQUIRE_DEVICE("c6_forward_generic");
   return launch_generic(x, x_dtype, batch, board, layers, kernels, channels, conv_w, conv_b,
                         pol_w, pol_b, val_w, val_b, prec, workspace, logits, value, mask_mode,
                         legal, fill, static_cast<hipStream_t>(stream));
@@ -294,6 +334,7 @@ int c6_mask_logits(const void *logits, const uint8_t *legal, int dtype, int64_t 
     set_error("c6_mask_logits: logits/out must be 16-byte and legal 8-byte aligned");
     return C6_EINVAL;
   }
+  C6_REQUIRE_DEVICE("c6_mask_logits");
   return launch_mask(logits, legal, eb, (long long)batch * C6_ACTIONS, fill_bits, out,
                      static_cast<hipStream_t>(stream));
 }
@@ -310,6 +351,7 @@ int c6_softmax_sample(const float *logits, const uint8_t *legal, const float *u,
     return C6_EINVAL;
   }
   const float inv_t = 1.0f / (temperature > 1e-4f ? temperature : 1e-4f);
+  C6_REQUIRE_DEVICE("c6_softmax_sample");
   return launch_sample(logits, legal, u, inv_t, batch, reinterpret_cast<long long *>(actions),
                        logprob, static_cast<hipStream_t>(stream));
 }
@@ -344,6 +386,8 @@ int c6_env_step(int8_t *boards, int8_t *current_player, int8_t *stones_left, int
   p.winner = winner;
   p.sign = transition_sign;
   p.lengths = game_lengths;
+  if (num_envs == 0) return C6_OK;
+  C6_REQUIRE_DEVICE("c6_env_step");
   return launch_env_step(p, static_cast<hipStream_t>(stream));
 }
 
@@ -359,6 +403,8 @@ int c6_canonical_input(const int8_t *boards, const int8_t *current_player,
     set_error("c6_canonical_input: null pointer");
     return C6_EINVAL;
   }
+  if (num_envs == 0) return C6_OK;
+  C6_REQUIRE_DEVICE("c6_canonical_input");
   return launch_canonical_input(boards, current_player, stones_left, num_envs, board_size, out,
                                 static_cast<hipStream_t>(stream));
 }
@@ -374,6 +420,7 @@ int c6_d4_expand(const void *x, int dtype, int64_t batch, void *out, void *strea
     set_error("c6_d4_expand: null pointer");
     return C6_EINVAL;
   }
+  C6_REQUIRE_DEVICE("c6_d4_expand");
   return launch_d4_expand(x, eb, batch, out, static_cast<hipStream_t>(stream));
 }
 
@@ -388,6 +435,7 @@ int c6_d4_reduce(const float *view_logits, const float *view_values, int64_t bat
     set_error("c6_d4_reduce: null pointer");
     return C6_EINVAL;
   }
+  C6_REQUIRE_DEVICE("c6_d4_reduce");
   return launch_d4_reduce(view_logits, view_values, batch, logits, values,
                           static_cast<hipStream_t>(stream));
 }

@@ -123,7 +123,7 @@ constexpr int kLoRing = 3;            // low-order weight prefetch ring depth (6
 // channels form a block follows from which lane holds them after the MFMA (lo6_channel).
 __host__ __device__ constexpr int lo6_channel(int cin, int block, int slot) {
   const int i = slot >> 1, odd = slot & 1;
-  int t, hh;
+  int t = 0, hh = 0;
   if (cin == 32) {          // one block: both lane halves of cout tile 0, gathered in one lane
     t = 0, hh = odd;
   } else if (block < 2) {   // block = lane half; even slots cout tile 0, odd slots cout tile 1

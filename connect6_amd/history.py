@@ -35,11 +35,29 @@ def _normalized_model_cfg(cfg: dict[str, Any]) -> dict[str, Any]:
     return out
 
 
+# bfloat16 selects the corrected bf16 mode (bf16 MFMA + fp6 pass on what the activations'
+# rounding dropped), the fastest bf16 mode that keeps >= 99 % of the fp32 argmax; the literal
+# "round every activation to bf16" arithmetic stays available as precision="bf16".
 _PREC_OF_DTYPE = {
     torch.float32: _lib.PREC_F32,
-    torch.bfloat16: _lib.PREC_BF16,
+    torch.bfloat16: _lib.PREC_BF16F6,
     torch.float16: _lib.PREC_F16,
 }
+
+
+def history_dtype(device: torch.device, dtype_name: str) -> torch.dtype:
+    """Ensemble dtype from the config's ``historical_inference_dtype``
+    (connect6/train.py:133-145): always float32 off the GPU, else by name."""
+    if torch.device(device).type != "cuda":
+        return torch.float32
+    name = dtype_name.lower()
+    if name == "bfloat16":
+        return torch.bfloat16
+    if name == "float16":
+        return torch.float16
+    if name == "float32":
+        return torch.float32
+    raise ValueError("historical_inference_dtype must be one of: bfloat16 | float16 | float32")
 
 
 class HistoricalPolicyEnsemble:
@@ -48,7 +66,13 @@ class HistoricalPolicyEnsemble:
     Input ``[MODELS, TABLES, 3, H, W]`` -> policy logits ``[MODELS, TABLES,
     H*W]`` in the ensemble dtype.  ``dtype`` selects the arithmetic as in the
     reference's ``_history_dtype`` (connect6/train.py:133-145): float32,
-    bfloat16 or float16.  ``precision`` may override it with ``"bf16x2"``.
+    bfloat16 or float16.  bfloat16 runs the corrected bf16 arithmetic
+    (``"bf16f6"``); ``precision`` may name any other mode, e.g. ``"bf16"``
+    for the literal bf16 rounding of every activation.
+
+    ``conv_weights``, ``conv_biases``, ``policy_weight`` and ``policy_bias``
+    (the reference's stacked ``[M, ...]`` tensors, connect6/history.py:224-233)
+    are built on first access: the forward reads only the packed copy.
     """
 
     def __init__(
@@ -81,19 +105,39 @@ class HistoricalPolicyEnsemble:
                 raise ValueError("historical checkpoints have different CNN architectures")
 
         states = [cp.model_state for cp in checkpoints]
-        # same attributes as the reference (history.py:224-233), on `device` in `dtype`
-        self.conv_weights: list[torch.Tensor] = []
-        self.conv_biases: list[torch.Tensor | None] = []
-        for i in range(len(self.kernels)):
-            self.conv_weights.append(self._stack(states, f"convs.{i}.weight"))
-            self.conv_biases.append(self._stack_optional(states, f"convs.{i}.bias"))
-        self.policy_weight = self._stack(states, "policy_output.weight")
-        self.policy_bias = self._stack_optional(states, "policy_output.bias")
+        required = [f"convs.{i}.weight" for i in range(len(self.kernels))] + ["policy_output.weight"]
+        for key in required:  # the KeyError of the reference's _stack (history.py:235-240)
+            for state in states:
+                if key not in state:
+                    raise KeyError(f"parameter {key} is missing from the historical checkpoints")
         self.action_size = self.board_size * self.board_size
 
         self._prec = _PREC_OF_DTYPE[self.dtype] if precision is None else _lib.PREC_BY_NAME[precision]
         self._packed: torch.Tensor | None = None
         self._states = states
+        self._stacked: dict[str, torch.Tensor | None] = {}
+
+    # -- the reference's stacked attributes, on `device` in `dtype`, built when first read --
+    def _stacked_attr(self, key: str, optional: bool) -> torch.Tensor | None:
+        if key not in self._stacked:
+            self._stacked[key] = (self._stack_optional if optional else self._stack)(self._states, key)
+        return self._stacked[key]
+
+    @property
+    def conv_weights(self) -> list[torch.Tensor]:
+        return [self._stacked_attr(f"convs.{i}.weight", False) for i in range(len(self.kernels))]
+
+    @property
+    def conv_biases(self) -> list[torch.Tensor | None]:
+        return [self._stacked_attr(f"convs.{i}.bias", True) for i in range(len(self.kernels))]
+
+    @property
+    def policy_weight(self) -> torch.Tensor:
+        return self._stacked_attr("policy_output.weight", False)
+
+    @property
+    def policy_bias(self) -> torch.Tensor | None:
+        return self._stacked_attr("policy_output.bias", True)
 
     def _stack(self, states, key: str) -> torch.Tensor:
         try:
@@ -117,15 +161,10 @@ class HistoricalPolicyEnsemble:
 
     def _model_state(self, m: int) -> dict[str, torch.Tensor]:
         """Parameters of model ``m`` as the ensemble holds them (rounded to ``dtype``)."""
-        state = {}
-        for i in range(len(self.kernels)):
-            state[f"convs.{i}.weight"] = self.conv_weights[i][m]
-            if self.conv_biases[i] is not None:
-                state[f"convs.{i}.bias"] = self.conv_biases[i][m]
-        state["policy_output.weight"] = self.policy_weight[m]
-        if self.policy_bias is not None:
-            state["policy_output.bias"] = self.policy_bias[m]
-        return state
+        keys = [f"convs.{i}.{kind}" for i in range(len(self.kernels)) for kind in ("weight", "bias")]
+        keys += ["policy_output.weight", "policy_output.bias"]
+        src = self._states[m]
+        return {k: src[k].detach().to(device=self.device, dtype=self.dtype) for k in keys if k in src}
 
     def _packed_weights(self) -> torch.Tensor:
         if self._packed is None:

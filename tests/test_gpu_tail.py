@@ -70,15 +70,17 @@ def test_sample_edge_cases(cuda):
     assert torch.allclose(lp.cpu(), torch.log(torch.tensor([1.0, 1.0, 0.5, 1 / 361])), atol=1e-5)
 
 
-def test_fused_selfplay_step_cfg4(cuda):
-    """B=16384, stones 0..300: forward + mask + softmax + draw in one launch."""
+@pytest.mark.parametrize("prec", ["bf16f6", "bf16x2"])
+def test_fused_selfplay_step_cfg4(cuda, prec):
+    """B=16384, stones 0..300: forward + mask + softmax + draw in one launch, in the headline
+    arithmetic mode (the one the benchmark times) and in the hi+lo bf16 mode."""
     b = 16384
     st = R.init_state(1234, "reference")
     x, legal = gen_boards(b, 300, 2025)
     u = gen_uniform(b, 7)
     model = c6.PolicyValueNet().to(cuda).eval()
     model.load_state_dict(st)
-    model.precision = "bf16x2"
+    model.precision = prec
     with torch.inference_mode():
         actions, logprob, value, masked = model.selfplay_step(x.to(cuda), u.to(cuda), 1.0, return_logits=True)
         a2, lp2, v2 = model.selfplay_step(x.to(cuda), u.to(cuda), 1.0)
@@ -98,6 +100,11 @@ def test_fused_selfplay_step_cfg4(cuda):
     a_ref, lp_ref = R.sample_inverse_cdf(lo, legal[:256], u[:256], 0.8)
     assert float((a4.cpu() == a_ref).float().mean()) >= 0.98   # logits differ by ~1e-6 relative
     assert rel_l2(v4, vo) <= 1e-4
+    # the 16-bit mode's own logits and value against the fp32 oracle on a slice the CPU does quickly
+    with torch.inference_mode():
+        lo2, vo2 = R.forward(st, x[:1024])
+    assert rel_l2(plain[:1024].cpu()[legal[:1024]], lo2[legal[:1024]]) <= 2e-2
+    assert rel_l2(value[:1024], vo2) <= 2e-2
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -123,7 +130,8 @@ def test_d4_reduce_matches_oracle(cuda):
     assert none is None and torch.equal(only, logits)
 
 
-def test_d4_evaluation_cfg5(cuda):
+@pytest.mark.parametrize("prec", ["bf16f6", "bf16x2"])
+def test_d4_evaluation_cfg5(cuda, prec):
     st = R.init_state(1234, "reference")
     model = c6.PolicyValueNet().to(cuda).eval()
     model.load_state_dict(st)
@@ -137,16 +145,21 @@ def test_d4_evaluation_cfg5(cuda):
     assert rel_l2(lg, lo) <= 1e-4 and rel_l2(vg, vo) <= 1e-4
     # full size (8192 base boards -> 65536 views) through a size-independent property:
     # the D4 average is invariant to presenting the board in another orientation
-    model.precision = "bf16x2"
+    model.precision = prec
     x, _ = gen_boards(8192, 200, 2025)
     xd = x.to(cuda)
     with torch.inference_mode():
         base_l, base_v = c6.evaluate_d4(model, xd)
         k, flip = R.symmetry_for_phase(5)
         rot_l, rot_v = c6.evaluate_d4(model, c6.transform_boards(xd, k, flip).contiguous())
+        # ... and a slice of the 16-bit result against the fp32 oracle pipeline
+        views = R.d4_expand(x[:128])
+        lv, vv = R.forward(st, views.reshape(8 * 128, 3, 19, 19))
+        lo, vo = R.d4_average(lv.view(8, 128, 361), vv.view(8, 128))
     a = torch.arange(361, device=cuda)
     back = rot_l[:, c6.transform_actions(a, 19, k, flip)]
     assert torch.allclose(back, base_l, atol=1e-6) and torch.allclose(rot_v, base_v, atol=1e-6)
+    assert rel_l2(base_l[:128], lo) <= 2e-2 and rel_l2(base_v[:128], vo) <= 2e-2
 
 
 def _random_states(n, seed):

@@ -24,6 +24,35 @@ def test_library_exports_every_declared_symbol():
     assert lib.c6_version() == 1
 
 
+def test_fused_kernels_stay_within_their_scratch_budget():
+    """One wave per SIMD: every scratch access of the fused kernel is latency next to the MFMAs.
+    The compiler's report from the last build bounds the spill bytes per lane of each
+    arithmetic mode (headline and plain 16-bit modes tight, the others a ceiling)."""
+    usage = _lib.resource_usage()
+    fused = {name: u for name, u in usage.items() if "fused_forward_kernel" in name}
+    assert len(fused) == 6
+    limit = {"PrecBF16F6": 64, "PrecBF16E": 52, "PrecF16": 52, "PrecBF16F8": 128, "PrecF32": 144, "PrecBF16X2": 256}
+    seen = set()
+    for name, u in fused.items():
+        for tag, cap in limit.items():
+            if tag in name:
+                seen.add(tag)
+                assert u["ScratchSize"] <= cap, (name, u)
+                assert u["VGPRs"] <= 256 and u["AGPRs"] <= 256 and u["Occupancy"] >= 1
+    assert seen == set(limit)
+
+
+def test_history_dtype_follows_the_reference_policy():
+    # connect6/train.py:133-145
+    cpu, gpu = torch.device("cpu"), torch.device("cuda", 0)
+    assert c6.history_dtype(cpu, "bfloat16") is torch.float32
+    assert c6.history_dtype(gpu, "bfloat16") is torch.bfloat16
+    assert c6.history_dtype(gpu, "Float16") is torch.float16
+    assert c6.history_dtype(gpu, "float32") is torch.float32
+    with pytest.raises(ValueError):
+        c6.history_dtype(gpu, "int8")
+
+
 def test_packed_sizes_follow_the_layout():
     # 1 KiB fragments: first layer 35 rows x (24/E) per half, 3x3 layers 9*Cin/KSTEP x Cout/32
     def frags(e):
@@ -165,7 +194,11 @@ def test_precision_resolution_follows_torch_rules():
     model.precision = "bf16x2"
     assert model.resolve_precision() == _lib.PREC_BF16X2
     model.precision = None
-    assert model.to(torch.bfloat16).resolve_precision() == _lib.PREC_BF16
+    # bf16 parameters (or bf16 autocast) select the corrected bf16 mode; plain bf16 is by name only
+    assert model.to(torch.bfloat16).resolve_precision() == _lib.PREC_BF16F6
+    assert model.to(torch.float16).resolve_precision() == _lib.PREC_F16
+    model.precision = "bf16"
+    assert model.resolve_precision() == _lib.PREC_BF16
 
 
 def test_mask_logits_argument_checks():
@@ -195,6 +228,10 @@ def test_history_ensemble_construction_and_validation():
     assert ens.conv_weights[0].shape == (2, 32, 3, 23, 23)
     assert ens.conv_biases[7].shape == (2, 96)
     assert ens.policy_weight.shape == (2, 1, 96, 1, 1) and ens.policy_bias.shape == (2, 1)
+    assert ens._prec == _lib.PREC_F32
+    ens16 = c6.HistoricalPolicyEnsemble(cps, torch.device("cpu"), dtype=torch.bfloat16)
+    assert ens16._prec == _lib.PREC_BF16F6 and ens16.conv_weights[3].dtype == torch.bfloat16
+    assert c6.HistoricalPolicyEnsemble(cps, torch.device("cpu"), dtype=torch.bfloat16, precision="bf16")._prec == _lib.PREC_BF16
     # compile keys are ignored when comparing architectures (history.py:69-73)
     cps[1].model_config["compile"] = True
     c6.HistoricalPolicyEnsemble(cps, torch.device("cpu"))
