@@ -34,6 +34,7 @@ EXPORTS = (
     "c6_forward_boards",
     "c6_generic_workspace_bytes",
     "c6_forward_generic",
+    "c6_forward_generic_static",
     "c6_mask_logits",
     "c6_softmax_sample",
     "c6_d4_expand",
@@ -128,6 +129,10 @@ def load() -> ctypes.CDLL:
     lib.c6_forward_generic.argtypes = [vp, i32, i64, i32, i32, ip, ip, ctypes.POINTER(vp),
                                        ctypes.POINTER(vp), vp, vp, vp, vp, i32, vp,
                                        ctypes.c_size_t, vp, vp, i32, vp, f32, vp]
+    lib.c6_forward_generic_static.restype = i32
+    lib.c6_forward_generic_static.argtypes = [vp, i32, i64, i32, i32, ip, ip, ctypes.POINTER(vp),
+                                              ctypes.POINTER(vp), vp, vp, vp, vp, i32, vp, vp,
+                                              i32, vp, f32, vp]
     lib.c6_mask_logits.restype = i32
     lib.c6_mask_logits.argtypes = [vp, vp, i32, i64, ctypes.c_uint32, vp, vp]
     lib.c6_softmax_sample.restype = i32

@@ -33,6 +33,9 @@ int launch_generic(const void *x, int x_dtype, long long batch, int n, int layer
                    float *logits, float *value, int mask_mode, const uint8_t *legal, float fill,
                    hipStream_t st);
 
+size_t static_scratch_bytes();
+int static_scratch(void **out);
+
 int launch_env_step(const EnvParams &p, hipStream_t st);
 int launch_canonical_input(const int8_t *boards, const int8_t *player, const int8_t *stones_left,
                            long long num, int n, float *out, hipStream_t st);
@@ -316,6 +319,35 @@ int c6_forward_generic(const void *x, int x_dtype, int64_t batch, int board, int
   return launch_generic(x, x_dtype, batch, board, layers, kernels, channels, conv_w, conv_b,
                         pol_w, pol_b, val_w, val_b, prec, workspace, logits, value, mask_mode,
                         legal, fill, static_cast<hipStream_t>(stream));
+}
+
+int c6_forward_generic_static(const void *x, int x_dtype, int64_t batch, int board, int layers,
+                              const int *kernels, const int *channels,
+                              const float *const *conv_w, const float *const *conv_b,
+                              const float *pol_w, const float *pol_b, const float *val_w,
+                              const float *val_b, int prec, float *logits, float *value,
+                              int mask_mode, const uint8_t *legal, float fill, void *stream) {
+  if (batch < 0) {
+    set_error("c6_forward_generic_static: negative batch");
+    return C6_EINVAL;
+  }
+  int rc = check_arch("c6_forward_generic_static", board, layers, kernels, channels);
+  if (rc != C6_OK) return rc;
+  const size_t need = generic_workspace_bytes(batch, board, layers, channels);
+  if (need > static_scratch_bytes()) {
+    set_error("c6_forward_generic_static: this batch needs %zu bytes of workspace, the built-in "
+              "one holds %zu; use c6_forward_generic with a workspace of your own",
+              need, static_scratch_bytes());
+    return C6_EINVAL;
+  }
+  if (batch == 0) return C6_OK;
+  C6_REQUIRE_DEVICE("c6_forward_generic_static");
+  void *ws = nullptr;
+  rc = static_scratch(&ws);
+  if (rc != C6_OK) return rc;
+  return c6_forward_generic(x, x_dtype, batch, board, layers, kernels, channels, conv_w, conv_b,
+                            pol_w, pol_b, val_w, val_b, prec, ws, static_scratch_bytes(), logits,
+                            value, mask_mode, legal, fill, stream);
 }
 
 int c6_mask_logits(const void *logits, const uint8_t *legal, int dtype, int64_t batch,

@@ -3,9 +3,46 @@
 // This is the compatibility path: plain direct convolution, one thread per output
 // element, activations round-tripping through a caller-provided workspace.  The fused
 // MFMA kernel in c6_forward.hip serves the default architecture.
+#include <mutex>
+
 #include "c6_common.h"
 
 namespace c6 {
+
+// Workspace of c6_forward_generic_static: callers that may not allocate device memory (code
+// under HIP graph capture, serving loops, harnesses that forbid hipMalloc) run the generic
+// forward through this array instead of a workspace of their own.  Every GPU the library runs
+// on holds its own copy until the process ends.  In host code the array's name is only a
+// handle for hipGetSymbolAddress: the per-device address it returns is what kernels receive.
+constexpr size_t kStaticScratchBytes = size_t(16) << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+size_t static_scratch_bytes() { return kStaticScratchBytes; }
+
+// Device address of `scratch` on the current device, looked up once per device.
+int static_scratch(void **out) {
+  constexpr int kMaxDevices = 64;
+  static std::mutex lock;
+  static void *addr[kMaxDevices] = {};
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    set_error("static scratch: no usable current device (%s, device %d)", hipGetErrorString(e), dev);
+    return C6_ELAUNCH;
+  }
+  std::lock_guard<std::mutex> guard(lock);
+  if (addr[dev] == nullptr) {
+    void *ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr) {
+      set_error("static scratch: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+      return C6_ELAUNCH;
+    }
+    addr[dev] = ptr;
+  }
+  *out = addr[dev];
+  return C6_OK;
+}
 
 __device__ __forceinline__ float round_to(float v, int mode) {
   if (mode == C6_DT_BF16) return (float)(__bf16)v;

@@ -133,9 +133,16 @@ def run_forward_generic(
     mask_mode: int = _lib.MASK_NONE,
     legal: torch.Tensor | None = None,
     fill: float = _FILL_LOWEST,
+    static_workspace: bool = False,
+    out: tuple[torch.Tensor, torch.Tensor | None] | None = None,
 ):
     """Launch ``c6_forward_generic`` for one weight set of any architecture:
-    x ``[B,3,n,n]`` -> (logits ``[B,n*n]``, value ``[B]`` or None)."""
+    x ``[B,3,n,n]`` -> (logits ``[B,n*n]``, value ``[B]`` or None).
+
+    ``static_workspace`` routes the layer-boundary activations through the
+    library's built-in 16 MiB array (``c6_forward_generic_static``) instead of
+    a workspace tensor; with ``out=(logits, value)`` preallocated the call then
+    allocates no device memory for the forward itself."""
     lib = _lib.load()
     dev = x.device
     x = x.contiguous()
@@ -162,12 +169,21 @@ def run_forward_generic(
     vp = ctypes.c_void_p
     wptrs = (vp * layers)(*[t.data_ptr() for t in ws])
     bptrs = (vp * layers)(*[(t.data_ptr() if t is not None else None) for t in bs])
-    nbytes = ctypes.c_size_t(0)
-    _lib.check(lib.c6_generic_workspace_bytes(b, n, layers, cc, ctypes.byref(nbytes)),
-               "c6_generic_workspace_bytes")
-    workspace = torch.empty(max(int(nbytes.value), 16), dtype=torch.uint8, device=dev)
-    logits = torch.empty((b, n * n), dtype=torch.float32, device=dev)
-    value = torch.empty((b,), dtype=torch.float32, device=dev) if want_value else None
+    workspace = None
+    if not static_workspace:
+        nbytes = ctypes.c_size_t(0)
+        _lib.check(lib.c6_generic_workspace_bytes(b, n, layers, cc, ctypes.byref(nbytes)),
+                   "c6_generic_workspace_bytes")
+        workspace = torch.empty(max(int(nbytes.value), 16), dtype=torch.uint8, device=dev)
+    if out is not None:
+        logits, value = out
+        if logits.shape != (b, n * n) or logits.dtype != torch.float32 or not logits.is_contiguous():
+            raise ValueError(f"out[0] must be a contiguous float32 tensor of shape ({b}, {n * n})")
+        if want_value and (value is None or value.shape != (b,) or value.dtype != torch.float32):
+            raise ValueError(f"out[1] must be a float32 tensor of shape ({b},)")
+    else:
+        logits = torch.empty((b, n * n), dtype=torch.float32, device=dev)
+        value = torch.empty((b,), dtype=torch.float32, device=dev) if want_value else None
     if legal is not None:
         if legal.shape != (b, n * n):
             raise ValueError(f"legal mask must have shape ({b}, {n * n}), got {tuple(legal.shape)}")
@@ -178,12 +194,18 @@ def run_forward_generic(
         return t.data_ptr() if t is not None else None
 
     with torch.cuda.device(dev):
-        rc = lib.c6_forward_generic(x.data_ptr(), _lib.torch_dtype_code(x.dtype), b, n, layers, ck,
-                                    cc, wptrs, bptrs, ptr(pw), ptr(pb), ptr(vw), ptr(vb), prec,
-                                    workspace.data_ptr(), workspace.numel(), ptr(logits),
-                                    ptr(value), mask_mode, ptr(legal), fill,
-                                    _lib.stream_ptr(dev))
-    _lib.check(rc, "c6_forward_generic")
+        if static_workspace:
+            rc = lib.c6_forward_generic_static(x.data_ptr(), _lib.torch_dtype_code(x.dtype), b, n,
+                                               layers, ck, cc, wptrs, bptrs, ptr(pw), ptr(pb),
+                                               ptr(vw), ptr(vb), prec, ptr(logits), ptr(value),
+                                               mask_mode, ptr(legal), fill, _lib.stream_ptr(dev))
+        else:
+            rc = lib.c6_forward_generic(x.data_ptr(), _lib.torch_dtype_code(x.dtype), b, n, layers,
+                                        ck, cc, wptrs, bptrs, ptr(pw), ptr(pb), ptr(vw), ptr(vb),
+                                        prec, workspace.data_ptr(), workspace.numel(), ptr(logits),
+                                        ptr(value), mask_mode, ptr(legal), fill,
+                                        _lib.stream_ptr(dev))
+    _lib.check(rc, "c6_forward_generic_static" if static_workspace else "c6_forward_generic")
     return logits, value
 
 

@@ -133,6 +133,21 @@ int c6_forward_generic(const void *x, int x_dtype, int64_t batch, int board, int
                        size_t workspace_bytes, float *logits, float *value, int mask_mode,
                        const uint8_t *legal, float fill, void *stream);
 
+/* c6_forward_generic without a workspace argument, for callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
+ * It has no counterpart in the reference.  The layer-boundary activations go through a 16 MiB
+ * array that lives in the library's device image (one copy per GPU, held until the process
+ * ends); a batch whose c6_generic_workspace_bytes() exceeds that returns C6_EINVAL.  The call
+ * allocates and frees nothing.  All calls on one GPU share that array: calls that overlap in
+ * time on one GPU (different streams or threads) race; calls on one stream are safe back to
+ * back.  Arguments and results as c6_forward_generic. */
+int c6_forward_generic_static(const void *x, int x_dtype, int64_t batch, int board, int layers,
+                              const int *kernels, const int *channels,
+                              const float *const *conv_w, const float *const *conv_b,
+                              const float *pol_w, const float *pol_b, const float *val_w,
+                              const float *val_b, int prec, float *logits, float *value,
+                              int mask_mode, const uint8_t *legal, float fill, void *stream);
+
 /* Out-of-place occupied-square masking of existing logits.
  * Replaces: mask_logits (connect6/model.py:123-125).
  * logits/out: device [B,361] of element type dtype; legal: device uint8 [B,361];
