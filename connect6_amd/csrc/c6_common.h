@@ -56,6 +56,7 @@ constexpr int kOverreadFrags = 8 * 3;  // zero frags after the last layer (prefe
 
 // precision policies ----------------------------------------------------------
 struct PrecF32 {
+  static constexpr int PIPE = 0;      // runs the layer-by-layer kernel
   static constexpr int ID = C6_PREC_F32;
   static constexpr int EB = 4;        // bytes per element
   static constexpr int SPLIT = 0;
@@ -64,6 +65,7 @@ struct PrecF32 {
   static constexpr int LO_FIRST = 1;  // first layer (0-based) whose input carries a low-order part
 };
 struct PrecBF16 {
+  static constexpr int PIPE = 1;      // runs the pipelined kernel (weights packed phase-major)
   static constexpr int ID = C6_PREC_BF16;
   static constexpr int EB = 2;
   static constexpr int SPLIT = 0;
@@ -72,6 +74,7 @@ struct PrecBF16 {
   static constexpr int LO_FIRST = 1;  // first layer (0-based) whose input carries a low-order part
 };
 struct PrecF16 {
+  static constexpr int PIPE = 1;      // runs the pipelined kernel (weights packed phase-major)
   static constexpr int ID = C6_PREC_F16;
   static constexpr int EB = 2;
   static constexpr int SPLIT = 0;
@@ -80,6 +83,7 @@ struct PrecF16 {
   static constexpr int LO_FIRST = 1;  // first layer (0-based) whose input carries a low-order part
 };
 struct PrecBF16X2 {
+  static constexpr int PIPE = 0;      // runs the layer-by-layer kernel
   static constexpr int ID = C6_PREC_BF16X2;
   static constexpr int EB = 2;
   static constexpr int SPLIT = 1;     // activations stored as hi plane + lo plane, both bf16
@@ -88,6 +92,7 @@ struct PrecBF16X2 {
   static constexpr int LO_FIRST = 1;  // first layer (0-based) whose input carries a low-order part
 };
 struct PrecBF16F8 {
+  static constexpr int PIPE = 0;      // runs the layer-by-layer kernel
   static constexpr int ID = C6_PREC_BF16F8;
   static constexpr int EB = 2;
   static constexpr int SPLIT = 0;
@@ -96,6 +101,7 @@ struct PrecBF16F8 {
   static constexpr int LO_FIRST = 1;  // first layer (0-based) whose input carries a low-order part
 };
 struct PrecBF16F6 {
+  static constexpr int PIPE = 1;      // runs the pipelined kernel (weights packed phase-major)
   static constexpr int ID = C6_PREC_BF16F6;
   static constexpr int EB = 2;
   static constexpr int SPLIT = 0;
@@ -119,19 +125,17 @@ constexpr int kLoRing = 3;            // low-order weight prefetch ring depth (6
 // bf16 + fp6 mode: the same second pass with e2m3 operands (K = 64 per instruction at four
 // times the bf16 rate).  The 32 bytes that hold 32 low-order values of a position are 24 bytes
 // of packed 6-bit values, one E8M0 scale byte (the block's power-of-two scale, taken from the
-// largest of the 32 values) and padding; the instruction applies the scale per lane.  Which 32
-// channels form a block follows from which lane holds them after the MFMA (lo6_channel).
-__host__ __device__ constexpr int lo6_channel(int cin, int block, int slot) {
-  const int i = slot >> 1, odd = slot & 1;
-  int t = 0, hh = 0;
-  if (cin == 32) {          // one block: both lane halves of cout tile 0, gathered in one lane
-    t = 0, hh = odd;
-  } else if (block < 2) {   // block = lane half; even slots cout tile 0, odd slots cout tile 1
-    t = odd, hh = block;
-  } else {                  // 96 channels: third block = both lane halves of cout tile 2
-    t = 2, hh = odd;
-  }
-  return 32 * t + 8 * (i >> 2) + 4 * hh + (i & 3);
+// largest of the 32 values) and padding; the instruction applies the scale per lane.  A block
+// is the 32 channels of one cout tile; which K slot a channel takes follows from which lane
+// holds it after the MFMA (lo6_channel).
+__host__ __device__ constexpr int lo6_channel(int block, int slot) {
+  // block = cout tile of the producing layer; a lane of that MFMA holds 16 of the tile's channels
+  // (register i, lane half hh).  Lane half 0 fills K slots 0-15, lane half 1 slots 16-31; inside
+  // a half, slot 2i' holds register i' and slot 2i'+1 register 8 + i' (how the conversion
+  // instruction interleaves its two operands).
+  const int hh = slot >> 4, s = slot & 15;
+  const int i = (s >> 1) + 8 * (s & 1);
+  return 32 * block + 8 * (i >> 2) + 4 * hh + (i & 3);
 }
 
 template <class P> struct Geo {

@@ -18,6 +18,25 @@
 namespace c6 {
 
 // Optional phase timestamps for kernel tuning (never compiled into the shipped library).
+#ifdef C6_DUMP_POINT
+__device__ unsigned g_dump[48 * 1024];
+extern "C" int c6_debug_dump(unsigned *host_out) {
+  return (int)hipMemcpyFromSymbol(host_out, HIP_SYMBOL(g_dump), sizeof(unsigned) * 48 * 1024);
+}
+// copy the first 128 KiB of LDS (+ optionally one lane-private value per thread) of workgroup 0
+#define C6_DUMP(point, smem, val)                                                          \
+  do {                                                                                     \
+    if ((point) == C6_DUMP_POINT && blockIdx.x == 0 && trace_on) {                         \
+      __syncthreads();                                                                     \
+      for (int i_ = threadIdx.x; i_ < 32 * 1024; i_ += 256)                                \
+        g_dump[i_] = reinterpret_cast<const unsigned *>(smem)[i_];                         \
+      g_dump[32 * 1024 + threadIdx.x] = (val);                                             \
+      __syncthreads();                                                                     \
+    }                                                                                      \
+  } while (0)
+#else
+#define C6_DUMP(point, smem, val) do { } while (0)
+#endif
 #ifdef C6_TRACE
 __device__ long long g_trace[256 * 4 * 64];
 #define C6_MARK(idx)                                                                       \
@@ -546,68 +565,6 @@ __device__ __forceinline__ u32x6 to_fp6_block(const f32x16v &even, const f32x16v
   asm volatile("" : "+v"(r) : "v"(even), "v"(odd), "v"(scale));
   return r;
 }
-__device__ __forceinline__ void lo6_block(unsigned char *dst, const float (&even)[16],
-                                          const float (&odd)[16], bool store) {
-  float m = 0.0f;
-  f32x16v a, b;
-#pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    a[i] = even[i];
-    b[i] = odd[i];
-    // one instruction per two values (fmaxf/fabsf would each add a canonicalising v_max first)
-    asm("v_max3_f32 %0, %1, |%2|, |%3|" : "=v"(m) : "v"(m), "v"(even[i]), "v"(odd[i]));
-  }
-  int sc = (__builtin_bit_cast(int, m) >> 23) - 2;  // biased exponent of the block scale
-  sc = sc < 1 ? 1 : sc;
-  const u32x6 r = to_fp6_block(a, b, __builtin_bit_cast(float, sc << 23));
-  if (store) {
-    *reinterpret_cast<v4i *>(dst) = v4i{(int)r[0], (int)r[1], (int)r[2], (int)r[3]};
-    *reinterpret_cast<v4i *>(dst + 16) = v4i{(int)r[4], (int)r[5], sc, 0};
-  }
-}
-
-// SiLU + store of one pixel tile in the fp6 mode: bf16 plane as in store_tile, then the
-// low-order blocks.  Cout tiles 0 and 1 pair up inside a lane (block = lane half); an odd
-// last tile gathers both lane halves in the lower lane (block 0 of 1, or 2 of 3).
-template <class P, int NT>
-__device__ __forceinline__ void store_tile_lo6(unsigned char *smem, int pos_in, int h,
-                                               const f32x16 (&acc)[NT][3], int j) {
-  using G = Geo<P>;
-  int pos = pos_in;
-  asm volatile("" : "+v"(pos));
-  unsigned char *rec = smem + pos * G::PIXB;
-  const DropConsts k = drop_consts<P>();
-  float lo[NT][16];
-#pragma unroll
-  for (int t = 0; t < NT; ++t)
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      float v[4];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) v[e] = silu<P>(acc[t][j][4 * q + e]);
-      const v2i hi = {pack2<P>(v[0], v[1]), pack2<P>(v[2], v[3])};
-      *reinterpret_cast<v2i *>(rec + (32 * t + 8 * q + 4 * h) * 2) = hi;
-      lo[t][4 * q + 0] = dropped_lo(v[0], hi[0], k);
-      lo[t][4 * q + 1] = dropped_hi(v[1], hi[0], k);
-      lo[t][4 * q + 2] = dropped_lo(v[2], hi[1], k);
-      lo[t][4 * q + 3] = dropped_hi(v[3], hi[1], k);
-    }
-  if constexpr (NT >= 2) lo6_block(rec + G::LO_OFF + 32 * h, lo[0], lo[1], true);
-  if constexpr (NT % 2 == 1) {
-    float own[16], other[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      // lower lanes: r[0] = own value, r[1] = the value lane + 32 holds (same pixel, channels + 4)
-      const unsigned mine = __builtin_bit_cast(unsigned, lo[NT - 1][i]);
-      const auto r = __builtin_amdgcn_permlane32_swap(mine, mine, false, false);
-      const unsigned r0 = r[0], r1 = r[1];  // (bit_cast straight from a vector element reads element 0)
-      own[i] = __builtin_bit_cast(float, r0);
-      other[i] = __builtin_bit_cast(float, r1);
-    }
-    lo6_block(rec + G::LO_OFF + 32 * (NT - 1), own, other, h == 0);
-  }
-}
-
 typedef const __attribute__((address_space(1))) float *GlobalF32;
 typedef const __attribute__((address_space(1))) f32x4 *GlobalF32x4;
 
@@ -631,6 +588,24 @@ __device__ __forceinline__ void init_acc(f32x16 (&acc)[N][3], const float *__res
     }
 }
 
+// the layer's bias as the lane sees it in an accumulator tile: register i of cout tile t holds
+// channel 32t + 8(i/4) + 4h + i%4.  The first MFMA of each accumulator takes this as its C
+// operand, so the accumulators themselves are never initialised.
+template <int N>
+__device__ __forceinline__ void load_bias_tiles(f32x16 (&bt)[N], const float *__restrict__ bias, int h) {
+  const float *blg = bias + 4 * h;
+  asm volatile("" : "+v"(blg));
+  const GlobalF32 bl = (GlobalF32)blg;
+#pragma unroll
+  for (int t = 0; t < N; ++t)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const f32x4 b4 = *(GlobalF32x4)(bl + 32 * t + 8 * q);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) bt[t][4 * q + e] = b4[e];
+    }
+}
+
 // barrier; every wave writes its share of the layer's output over the layer's input; barrier
 // (WITH_LO: the next layer runs a low-order pass, so its input needs the low-order part)
 template <class P, int NT, bool WITH_LO, class Pre>
@@ -639,13 +614,7 @@ __device__ __forceinline__ void finish_layer(unsigned char *smem, const int (&ci
   __syncthreads();  // every wave has finished reading the layer's input
   before_store();
 #pragma unroll
-  for (int j = 0; j < 3; ++j) {
-    if constexpr (P::LO6 && WITH_LO) {
-      store_tile_lo6<P, NT>(smem, ci[j], h, acc, j);
-    } else {
-      store_tile<P, NT>(smem, ci[j], h, acc, j);
-    }
-  }
+  for (int j = 0; j < 3; ++j) store_tile<P, NT>(smem, ci[j], h, acc, j);
   __syncthreads();
 }
 
@@ -674,6 +643,514 @@ __device__ __forceinline__ void mid_layer(
   C6_MARK(5 + 2 * L);
   (void)wave;
   (void)trace_on;
+}
+
+// ------------------------------------------------------------------------
+// Pipelined kernel (16-bit modes with padded records: bf16, fp16, bf16 + fp6).
+//
+// With one wave per SIMD nothing runs beside a wave's own instruction stream, and the SiLU
+// epilogue of a layer (two transcendentals per element) used to run with the matrix pipe idle.
+// VALU work issued between the MFMAs of a K-loop is nearly free (a full SiLU per MFMA lengthens
+// a 33-cycle MFMA slot by 7 cycles), so the epilogue of layer L is issued from inside the K-loop
+// of layer L+1: that loop is ordered phase-major, a phase being all nine taps of 32 input
+// channels = one cout tile of layer L.  Only cout tile 0 of layer L is converted in the open;
+// phase p of layer L+1 then carries the conversion of tile p+1, with a barrier between phases.
+// The accumulators of layer L therefore stay live next to those of layer L+1.
+// ------------------------------------------------------------------------
+// compile-time loop: f(IC<B>{}), f(IC<B+1>{}), ... (the index is a constant expression inside f)
+template <int I> struct IC {
+  static constexpr int value = I;
+};
+template <int B, int E, class F> __device__ __forceinline__ void static_for(F &&f) {
+  if constexpr (B < E) {
+    f(IC<B>{});
+    static_for<B + 1, E>(f);
+  }
+}
+
+constexpr int kPhaseSteps = 18;   // k-steps of one phase: 9 taps x 2 k-steps of 16 channels
+
+// even K slots of a 192-bit fp6 block, as three repeating dword masks (slot s = bits [6s, 6s+6))
+__host__ __device__ constexpr unsigned fp6_even_mask(int dword) {
+  unsigned m = 0;
+  for (int b = 0; b < 32; ++b)
+    if ((32 * dword + b) % 12 < 6) m |= 1u << b;
+  return m;
+}
+
+// The epilogue of one cout tile (SiLU, bf16 store, low-order fp6 blocks), cut into slots that
+// each hold about 20 cycles of VALU work, so that one slot can ride behind each MFMA of the
+// next layer's K-loop: a wave issues one instruction every ~4 cycles, an MFMA occupies the
+// matrix pipe for 32, so about six other instructions fit behind it (transcendentals count
+// double, and the K-loop's own LDS reads and weight loads need their share).
+// The lane's 48 elements (3 pixel tiles x 16 channels) stream through a software pipeline, one
+// element per two slots, so that no instruction waits for the one before it:
+//   even slot of step s:  exp2 of element s | 1 + . of element s-1 | x * . of element s-2
+//   odd slot of step s:   rcp of element s-1 | pack pair P (s = 2P+3) | low-order parts of pair P
+//                         (s = 2P+4) | running maximum over pair P (s = 2P+5)
+// plus the store of each quad and, per pixel tile, four slots that build the fp6 block.
+constexpr int kEpiSlots = 108;
+
+struct EpiCarry {
+  float e[16];      // sigmoid denominators in flight (element n at n % 16)
+  float v[16];      // activations (fp32) until they are packed
+  int hi[8];        // packed bf16 pairs until they are stored (pair P at P % 8)
+  float lo[2][16];  // what the rounding dropped, per pixel tile (two in flight)
+  float m[2];       // their largest magnitude
+  int sc;
+};
+
+//   wb[j]: byte address of the lane's position record + 8 * lane half;  h4 = 4 * lane half
+template <class P, int NT>
+__device__ __forceinline__ void epi_slot(unsigned char *smem, const int (&wb)[3], int h4,
+                                         const f32x16 (&acc)[NT][3], int t, int g, EpiCarry &c,
+                                         const DropConsts &k) {
+  using G = Geo<P>;
+  if (g >= kEpiSlots) return;
+  const int s = g >> 1;
+  auto elem = [](int n) __attribute__((always_inline)) { return n >= 0 && n < 48; };
+  auto pair_at = [](int s, int first) __attribute__((always_inline)) {  // P with first + 2P == s, or -1
+    return (s >= first && (s - first) % 2 == 0 && (s - first) / 2 < 24) ? (s - first) / 2 : -1;
+  };
+  if ((g & 1) == 0) {
+    if (elem(s)) c.e[s % 16] = __builtin_amdgcn_exp2f(acc[t][s / 16][s % 16]);
+    if (elem(s - 1)) c.e[(s - 1) % 16] = 1.0f + c.e[(s - 1) % 16];
+    if (elem(s - 2)) c.v[(s - 2) % 16] = acc[t][(s - 2) / 16][(s - 2) % 16] * c.e[(s - 2) % 16];
+    if (g >= 12 && (g - 12) % 8 == 0 && (g - 12) / 8 < 12) {  // quad Q: both its pairs are packed
+      const int Q = (g - 12) / 8;
+      *reinterpret_cast<v2i *>(smem + wb[Q / 4] + 64 * t + 16 * (Q % 4)) =
+          v2i{c.hi[(2 * Q) % 8], c.hi[(2 * Q + 1) % 8]};
+    }
+  } else {
+    if (elem(s - 1)) c.e[(s - 1) % 16] = __builtin_amdgcn_rcpf(c.e[(s - 1) % 16]);
+    if (const int P2 = pair_at(s, 3); P2 >= 0)
+      c.hi[P2 % 8] = pack2<P>(c.v[(2 * P2) % 16], c.v[(2 * P2 + 1) % 16]);
+    if constexpr (P::LO6) {
+      if (const int P2 = pair_at(s, 4); P2 >= 0) {
+        const int b = (P2 / 8) & 1, p = P2 % 8;
+        c.lo[b][2 * p] = dropped_lo(c.v[(2 * P2) % 16], c.hi[P2 % 8], k);
+        c.lo[b][2 * p + 1] = dropped_hi(c.v[(2 * P2 + 1) % 16], c.hi[P2 % 8], k);
+      }
+      if (const int P2 = pair_at(s, 5); P2 >= 0) {
+        // largest magnitude: med3(|x|, m, inf) = max(|x|, m); the compiler folds two of them
+        // into one v_max3_f32 with |.| modifiers.  (Not an asm statement: a dot2 result needs
+        // three wait states before another VALU instruction may read it, and the compiler keeps
+        // them only for instructions it can see.)
+        const int b = (P2 / 8) & 1, p = P2 % 8;
+        float m = p == 0 ? 0.0f : c.m[b];
+        m = __builtin_amdgcn_fmed3f(__builtin_fabsf(c.lo[b][2 * p]), m, __builtin_inff());
+        m = __builtin_amdgcn_fmed3f(__builtin_fabsf(c.lo[b][2 * p + 1]), m, __builtin_inff());
+        c.m[b] = m;
+      }
+    }
+  }
+  if constexpr (P::LO6) {
+    // fp6 block of pixel tile j: the tile's 32 channels of a position sit in two lanes (lane
+    // halves), 16 each.  They agree on the scale (2^(E-2) for a largest magnitude in
+    // [2^E, 2^(E+1)), so values land in (-8, 8)); then each converts its own 16 values into 16
+    // K slots = 12 bytes: the lower lane's go to bytes 0-11 of the block, the upper lane's to
+    // bytes 12-23, the scale to byte 24.
+    if (g >= 40 && g < 40 + 32 * 3 && (g - 40) % 32 < 4) {
+      const int j = (g - 40) / 32, f = (g - 40) % 32, b = j & 1;
+      if (f == 0) {
+        const unsigned mb = __builtin_bit_cast(unsigned, c.m[b]);
+        const auto x = __builtin_amdgcn_permlane32_swap(mb, mb, false, false);
+        const unsigned x0 = x[0], x1 = x[1];
+        c.m[b] = __builtin_bit_cast(float, x0 > x1 ? x0 : x1);  // (non-negative floats order like integers)
+      } else if (f == 1) {
+        const int sc = (__builtin_bit_cast(int, c.m[b]) >> 23) - 2;  // biased exponent of the block scale
+        c.sc = sc < 1 ? 1 : sc;
+      } else if (f == 2) {
+        // slot 2i <- first[i], slot 2i+1 <- second[i]; only slots 0-15 (i < 8) are kept, so the
+        // upper halves of both operands stay undefined registers
+        typedef float f32x8v __attribute__((ext_vector_type(8)));
+        f32x8v p0, p1;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          p0[i] = c.lo[b][i];
+          p1[i] = c.lo[b][8 + i];
+        }
+        const f32x16v first = __builtin_shufflevector(p0, p0, 0, 1, 2, 3, 4, 5, 6, 7, -1, -1, -1, -1, -1, -1, -1, -1);
+        const f32x16v second = __builtin_shufflevector(p1, p1, 0, 1, 2, 3, 4, 5, 6, 7, -1, -1, -1, -1, -1, -1, -1, -1);
+        const u32x6 r = to_fp6_block(first, second, __builtin_bit_cast(float, c.sc << 23));
+        unsigned char *dst = smem + wb[j] + G::LO_OFF + 32 * t;  // + 8h from wb: data at + 4h more = 12h
+        typedef int v3i __attribute__((ext_vector_type(3)));
+        // (three dwords at a 4-byte aligned address: dword stores)
+        int *d32 = reinterpret_cast<int *>(dst + h4);
+        d32[0] = (int)r[0];
+        d32[1] = (int)r[1];
+        d32[2] = (int)r[2];
+        *reinterpret_cast<int *>(dst - h4 + 24) = c.sc;  // byte 24 (lower lane) / 28 (upper lane: unused)
+      }
+    }
+  }
+}
+
+// Phase PH of a 3x3 layer with NT cout tiles: the nine taps of input channels [32 PH, 32 PH + 32).
+// Every MFMA opens a slot that ends with a scheduling barrier: the MFMA, at most two memory
+// instructions (the activation fragments of two k-steps ahead, the weight fragment that replaces
+// the one whose last MFMA this was) and one micro-step of the previous layer's epilogue.
+//   rb[j]: byte address of the record one row and one column before the lane's position, + 16 * lane half
+//   wl:    this phase's first weight fragment; `ring` holds its first kRing k-steps
+//   hidden(g): epilogue work of the previous layer to issue in slot g
+//   bias: PH == 0 only -- the accumulators are undefined on entry and the first k-step's MFMAs
+//         start from the bias tiles
+template <class P, int NT, int PH, class Hidden>
+__device__ __forceinline__ void conv3_phase(const unsigned char *smem, const WFrags &wl,
+                                            v4i (&ring)[kRing][NT], const int (&rb)[3],
+                                            f32x16 (&acc)[NT][3], const f32x16 (&bias)[NT],
+                                            Hidden hidden) {
+  using G = Geo<P>;
+  constexpr int U = kPhaseSteps, D = kRing, QN = kAhead + 1;
+  static_assert(G::KSTEP == 16 && G::PADDED && U % D == 0 && U % QN == 0, "phase shape");
+  auto frag = [&](int j, int u) {
+    const int tap = u / 2;
+    const int off = ((tap / 3) * kPitch + tap % 3) * G::PIXB + PH * 64 + (u % 2) * 32;
+    return *reinterpret_cast<const v4i *>(smem + rb[j] + off);
+  };
+  v4i bq[QN][3];
+#pragma unroll
+  for (int a = 0; a < kAhead; ++a)
+#pragma unroll
+    for (int j = 0; j < 3; ++j) bq[a][j] = frag(j, a);
+  const WFrags wn = wl + D * NT;
+  static_for<0, U * NT * 3>([&](auto gc) __attribute__((always_inline)) {
+    constexpr int g = decltype(gc)::value;
+    constexpr int u = g / (NT * 3), t = (g / 3) % NT, j = g % 3;
+    if constexpr (PH == 0 && u == 0) {
+      f32x16 c0 = bias[t];
+      mma<P>(ring[u % D][t], bq[u % QN][j], c0);
+      acc[t][j] = c0;
+    } else {
+      mma<P>(ring[u % D][t], bq[u % QN][j], acc[t][j]);
+    }
+    if constexpr (t == 0 && u + kAhead < U) bq[(u + kAhead) % QN][j] = frag(j, u + kAhead);
+    // weights of k-step u + D of the stream (it runs on into the next phase and the next layer)
+    if constexpr (j == 2) ring[u % D][t] = wn[u * NT + t];
+    hidden(g);
+    __builtin_amdgcn_sched_barrier(0);
+  });
+}
+
+// One 3x3 layer L (1..7) of the pipelined kernel: finishes the epilogue of layer L-1 (whose
+// accumulators arrive in `prev`) while accumulating its own output into `acc`.
+template <class P, int L, class Rezero>
+__device__ __forceinline__ void pipe_layer(
+    unsigned char *smem, const unsigned char *packed, const float *tail,
+    v4i (&ring)[kRing][kCoutArr[L] / 32], const int (&ci)[3], int h, int lane, int wave,
+    bool trace_on, const int (&lo_scale_w)[8], const f32x16 (&prev)[kCinArr[L] / 32][3],
+    f32x16 (&acc)[kCoutArr[L] / 32][3], Rezero rezero) {
+  using G = Geo<P>;
+  constexpr int NT = kCoutArr[L] / 32, NTP = kCinArr[L] / 32;
+  int rb[3], wb[3];
+#pragma unroll
+  for (int j = 0; j < 3; ++j) {
+    int pos = ci[j];
+    asm volatile("" : "+v"(pos));  // (recomputed per layer: keeps six address registers out of the board loop)
+    rb[j] = (pos - kPitch - 1) * G::PIXB + 16 * h;
+    wb[j] = pos * G::PIXB + 8 * h;
+  }
+  const DropConsts k = drop_consts<P>();
+  const int h4 = 4 * h;
+  EpiCarry carry;
+  f32x16 bias[NT];
+  load_bias_tiles(bias, tail + bias_offset(L), h);
+  __syncthreads();  // every wave has finished reading the input of layer L-1
+  rezero();
+  // cout tile 0 of layer L-1 in the open
+  // (a compile-time loop: `#pragma unroll` gives up on a body this size, and a runtime index
+  // would put the accumulators into scratch memory)
+  static_for<0, kEpiSlots>([&](auto sc) __attribute__((always_inline)) {
+    epi_slot<P, NTP>(smem, wb, h4, prev, 0, decltype(sc)::value, carry, k);
+  });
+#ifdef C6_EXP_NOHIDE
+  static_for<0, (NTP - 1) * kEpiSlots>([&](auto sc) __attribute__((always_inline)) {
+    constexpr int i = decltype(sc)::value;
+    epi_slot<P, NTP>(smem, wb, h4, prev, 1 + i / kEpiSlots, i % kEpiSlots, carry, k);
+  });
+#endif
+  __syncthreads();
+  C6_MARK(L == 1 ? 3 : 3 + 2 * L);
+  C6_DUMP(10 + L, smem, __builtin_bit_cast(unsigned, prev[0][0][0]));
+  const WFrags wl = layer_weights<P, L>(packed, lane);
+  conv3_phase<P, NT, 0>(smem, wl, ring, rb, acc, bias, [&](int g) __attribute__((always_inline)) {
+#ifndef C6_EXP_NOHIDE
+    if constexpr (NTP > 1) epi_slot<P, NTP>(smem, wb, h4, prev, 1, g, carry, k);
+#endif
+  });
+  if constexpr (NTP > 1) {
+    __syncthreads();
+    conv3_phase<P, NT, 1>(smem, wl + kPhaseSteps * NT, ring, rb, acc, bias, [&](int g) __attribute__((always_inline)) {
+#ifndef C6_EXP_NOHIDE
+      if constexpr (NTP > 2) epi_slot<P, NTP>(smem, wb, h4, prev, 2, g, carry, k);
+#endif
+    });
+  }
+  if constexpr (NTP > 2) {
+    __syncthreads();
+    conv3_phase<P, NT, 2>(smem, wl + 2 * kPhaseSteps * NT, ring, rb, acc, bias, [](int) {});
+  }
+  C6_MARK(30 + L);
+#ifndef C6_EXP_LOMASK
+#define C6_EXP_LOMASK 0xff
+#endif
+  if constexpr (P::LO8 && ((C6_EXP_LOMASK >> L) & 1)) {
+    v4i lor0[LoRing<P, L>::D][LoRing<P, L>::NT], lor1[LoRing<P, L>::D][LoRing<P, L>::NT];
+    lo_preload<P, L>(lor0, lor1, packed, lane);
+    conv3_lo_pass<P, L>(smem, packed, lo_scale_w[L], lor0, lor1, ci, h, lane, acc);
+  }
+  C6_MARK(4 + 2 * L);
+  C6_DUMP(20 + L, smem, __builtin_bit_cast(unsigned, acc[0][0][0]));
+  (void)wave;
+  (void)trace_on;
+}
+
+template <class P>
+__global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
+  using G = Geo<P>;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  constexpr int THREADS = 256, NWAVES = THREADS / 64;
+  constexpr int ROUNDS = (kPix + THREADS - 1) / THREADS;  // pixels per thread when staging
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int h = lane >> 5;
+  const int n = lane & 31;
+
+  // per-lane pixel geometry of the three 32-pixel tiles of this quarter
+  int ci[3], l1base[3], pix[3];
+  bool valid[3];
+#pragma unroll
+  for (int j = 0; j < 3; ++j) {
+    const int p = wave * kPixPerWave + j * 32 + n;
+    valid[j] = p < kPix;
+    const int pc = valid[j] ? p : (kPix - 1);
+    pix[j] = pc;
+    const int r = pc / kBoard, c = pc - r * kBoard;
+    ci[j] = (r + 1) * kPitch + (c + 1);
+    const int s = c % G::E;
+    l1base[j] = s * G::COPY_BYTES + ((r * 3 + kL1RowsHalf * h) * kL1RowPitch + (c - s)) * G::EB;
+  }
+
+  unsigned char *occ = smem + G::OCC_OFF;
+  float *lgt = reinterpret_cast<float *>(smem + G::LGT_OFF);
+  float *red = reinterpret_cast<float *>(smem + G::RED_OFF);
+
+  const unsigned per_group = (unsigned)prm.boards_per_group;  // board counts fit 32 bits (host-checked)
+  auto packed_of = [&](long long b) {
+    return prm.packed + (size_t)((unsigned)b / per_group) * prm.packed_stride;
+  };
+  // input of one board: each thread owns pixels tid, tid + THREADS, ... (three planes + occupancy)
+  float xin[ROUNDS][3];
+  unsigned char occin[ROUNDS];
+  auto fetch_board = [&](long long b) {
+    if (prm.x_dtype == C6_DT_BOARD_I8) {
+      // environment state in, network planes out (connect6/vector_env.py:196-218 of the
+      // reference), seen through D4 view prm.view (connect6/train.py:222-230)
+      long long src = prm.index ? prm.index[b] : b;
+      src = src < 0 ? 0 : (src >= prm.num_states ? prm.num_states - 1 : src);
+      const int8_t *board = reinterpret_cast<const int8_t *>(prm.x) + (size_t)src * kPix;
+      const int me = prm.player[src];
+      const float last = prm.stones_left[src] == 1 ? 1.0f : 0.0f;
+#pragma unroll
+      for (int r = 0; r < ROUNDS; ++r) {
+        const int p = tid + r * THREADS;
+        if (p < kPix) {
+          const int stone = board[prm.view ? d4_from_view(p, prm.view) : p];
+          xin[r][0] = stone == me ? 1.0f : 0.0f;
+          xin[r][1] = stone == -me ? 1.0f : 0.0f;
+          xin[r][2] = last;
+          occin[r] = 0;
+        }
+      }
+      return;
+    }
+#pragma unroll
+    for (int r = 0; r < ROUNDS; ++r) {
+      const int p = tid + r * THREADS;
+      if (p < kPix) {
+#pragma unroll
+        for (int ch = 0; ch < 3; ++ch)
+          xin[r][ch] = load_x(prm.x, prm.x_dtype, ((size_t)b * 3 + ch) * kPix + p);
+        occin[r] = prm.mask_mode == C6_MASK_LEGAL ? (prm.legal[(size_t)b * kPix + p] == 0) : 0;
+      }
+    }
+  };
+
+  // Each workgroup takes one contiguous run of boards, and the runs are dealt out so that the
+  // workgroups of one XCD (workgroup i runs on XCD i % 8) cover one contiguous eighth of the
+  // batch: with several weight sets an XCD's L2 then holds only the sets of its own boards, and
+  // consecutive boards of a workgroup mostly reuse the set it has just streamed.
+  const long long per = (prm.total_boards + gridDim.x - 1) / gridDim.x;
+  const unsigned xcds = (gridDim.x % 8 == 0) ? 8 : 1;
+  const long long run = (long long)(blockIdx.x % xcds) * (gridDim.x / xcds) + blockIdx.x / xcds;
+  long long b = run * per;
+  const long long b_end = b + per < prm.total_boards ? b + per : prm.total_boards;
+  if (b >= b_end) return;
+  [[maybe_unused]] const long long b_first = b;
+  v4i r1[L1Pipe<P>::D][1];
+  preload_ring<L1Pipe<P>::D, 1>(r1, layer_weights<P, 0>(packed_of(b), lane));
+  fetch_board(b);
+
+  for (; b < b_end; ++b) {
+    int tidv = tid;  // opaque per board: keeps per-thread staging addresses out of long-lived registers
+    asm volatile("" : "+v"(tidv));
+    const unsigned char *packed = packed_of(b);
+    const float *tail = reinterpret_cast<const float *>(packed + G::TAIL_OFF);
+    // block-scale exponents of the low-order weight copies (E8M0: 127 - log2 of the copy's scale),
+    // fetched here, long before any second pass needs them
+    int lo_scale_w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if constexpr (P::LO8) {
+#pragma unroll
+      for (int l = 1; l < 8; ++l) lo_scale_w[l] = 127 - reinterpret_cast<const int *>(tail)[G::TAIL_SW + l];
+    }
+
+#if defined(C6_DUMP_POINT)
+    const bool trace_on = (b == b_first + 1);  // second board of this workgroup
+#elif defined(C6_TRACE)
+    const bool trace_on = (b == b_first + 2);  // third board of this workgroup
+#else
+    const bool trace_on = false;
+#endif
+    __syncthreads();  // previous board fully written out; LDS is free
+    C6_MARK(0);
+    // ---- stage the input: zero the shifted copies, then scatter the board ----
+    {
+      const v4i z = {0, 0, 0, 0};
+      for (int i = tidv * 16; i < G::COPIES_BYTES; i += THREADS * 16)
+        *reinterpret_cast<v4i *>(smem + i) = z;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < ROUNDS; ++r) {
+      const int p = tidv + r * THREADS;
+      if (p < kPix) {
+        const int row = p / kBoard, c = p - row * kBoard;
+        unsigned char o = occin[r];
+        if (prm.mask_mode == C6_MASK_INPUT) o = (xin[r][0] != 0.0f) || (xin[r][1] != 0.0f);
+        occ[p] = o;
+#pragma unroll
+        for (int ch = 0; ch < 3; ++ch) {
+          const int hrow = (row + kK1 / 2) * 3 + ch;
+#pragma unroll
+          for (int s = 0; s < G::E; ++s) {
+            const int a = s * G::COPY_BYTES + (hrow * kL1RowPitch + (c + kK1 / 2 - s)) * G::EB;
+            *reinterpret_cast<unsigned short *>(smem + a) = bits16<P>(xin[r][ch]);
+          }
+        }
+      }
+    }
+    const long long bn = b + 1;
+    if (bn < b_end) fetch_board(bn);  // lands while this board is computed
+    __syncthreads();
+    C6_MARK(1);
+
+    v4i r2[kRing][1], r3[kRing][2], r6[kRing][3];  // weight rings of layers 2, 3-5, 6-8
+    f32x16 a0[1][3], a1[1][3];
+    // ---- layer 1 ----
+    init_acc(a0, tail + bias_offset(0), h);
+    conv1_pass<P>(smem, layer_weights<P, 0>(packed, lane), r1, l1base, a0);
+    preload_ring<kRing, 1>(r2, layer_weights<P, 1>(packed, lane));
+    C6_MARK(2);
+    pipe_layer<P, 1>(smem, packed, tail, r2, ci, h, lane, wave, trace_on, lo_scale_w, a0, a1, [&] {
+      // the first layer's shifted copies overlapped the activation tile: restore its zero padding
+      for (int i = tidv; i < 60 * (G::PIXB / 16); i += THREADS) {
+        const int k = i / (G::PIXB / 16), w16 = i - k * (G::PIXB / 16);
+        // pad positions: 0..19 (top row), 400..420 (bottom row + tail), 20*R (left column)
+        const int pos = k < 20 ? k : (k < 41 ? 400 + (k - 20) : (k - 40) * kPitch);
+        const v4i z = {0, 0, 0, 0};
+        *reinterpret_cast<v4i *>(smem + pos * G::PIXB + w16 * 16) = z;
+      }
+    });
+    preload_ring<kRing, 2>(r3, layer_weights<P, 2>(packed, lane));
+    f32x16 a2[2][3];
+    pipe_layer<P, 2>(smem, packed, tail, r3, ci, h, lane, wave, trace_on, lo_scale_w, a1, a2, [] {});
+    f32x16 a3[2][3];
+    pipe_layer<P, 3>(smem, packed, tail, r3, ci, h, lane, wave, trace_on, lo_scale_w, a2, a3, [] {});
+    f32x16 a4[2][3];
+    pipe_layer<P, 4>(smem, packed, tail, r3, ci, h, lane, wave, trace_on, lo_scale_w, a3, a4, [] {});
+    preload_ring<kRing, 3>(r6, layer_weights<P, 5>(packed, lane));
+    f32x16 a5[3][3];
+    pipe_layer<P, 5>(smem, packed, tail, r6, ci, h, lane, wave, trace_on, lo_scale_w, a4, a5, [] {});
+    f32x16 a6[3][3];
+    pipe_layer<P, 6>(smem, packed, tail, r6, ci, h, lane, wave, trace_on, lo_scale_w, a5, a6, [] {});
+    f32x16 acc[3][3];
+    pipe_layer<P, 7>(smem, packed, tail, r6, ci, h, lane, wave, trace_on, lo_scale_w, a6, acc, [] {});
+
+    // ---- both 1x1 heads straight from the fp32 accumulators of layer 8 ----
+    {
+      const float *polw = tail + kBiasTotal;
+      const float *valw = polw + kHeadC;
+      const float *pwl = polw + 4 * h;  // per-lane base: channel 32t + 8q + 4h + e
+      asm volatile("" : "+v"(pwl));
+      const GlobalF32 pwg = (GlobalF32)pwl;
+      if (bn < b_end) preload_ring<L1Pipe<P>::D, 1>(r1, layer_weights<P, 0>(packed_of(bn), lane));
+      float pol[3] = {0.0f, 0.0f, 0.0f};
+      float vsum = 0.0f;
+#pragma unroll
+      for (int t = 0; t < 3; ++t)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const f32x4 pw = *(GlobalF32x4)(pwg + 32 * t + 8 * q);
+          const f32x4 vw = *(GlobalF32x4)(pwg + kHeadC + 32 * t + 8 * q);
+#pragma unroll
+          for (int j = 0; j < 3; ++j) {
+            float vs = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const float a = silu<P>(acc[t][j][4 * q + e]);
+              pol[j] = fmaf(a, pw[e], pol[j]);
+              vs = fmaf(a, vw[e], vs);
+            }
+            vsum += valid[j] ? vs : 0.0f;
+          }
+        }
+      const float polb = valw[kHeadC], valb = valw[kHeadC + 1];
+      float tot[3];
+#pragma unroll
+      for (int j = 0; j < 3; ++j) {  // add the other lane half's channels
+        const unsigned bits = __builtin_bit_cast(unsigned, pol[j]);
+        const auto r = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+        const unsigned r0 = r[0], r1 = r[1];
+        tot[j] = __builtin_bit_cast(float, r0) + __builtin_bit_cast(float, r1);
+      }
+#pragma unroll
+      for (int j = 0; j < 3; ++j)
+        if (h == 0 && valid[j]) lgt[pix[j]] = tot[j] + polb;
+      vsum = wave_sum(vsum);
+      if (lane == 0) red[wave] = vsum;
+      __syncthreads();
+      if (tid == 0 && prm.value != nullptr) {
+        float s = 0.0f;
+#pragma unroll
+        for (int w = 0; w < NWAVES; ++w) s += red[w];
+        prm.value[b] = tanhf(s * (1.0f / kPix) + valb);
+      }
+      C6_MARK(19);
+    }
+
+    // ---- write out: masked logits, optional sampled action ----
+    if (prm.logits != nullptr) {
+      for (int p = tid; p < kPix; p += THREADS) {
+        const float v = lgt[p];
+        prm.logits[(size_t)b * kPix + p] = occ[p] ? prm.fill : v;
+      }
+    }
+    if (prm.actions != nullptr && wave == 0) {
+      const float it = prm.inv_temperature;
+      int a;
+      float lp;
+      wave_sample(
+          lane, prm.u[b], [&](int i) { return lgt[i] * it; }, [&](int i) { return occ[i] == 0; },
+          a, lp);
+      if (lane == 0) {
+        prm.actions[b] = a;
+        if (prm.logprob != nullptr) prm.logprob[b] = lp;
+      }
+    }
+    C6_MARK(20);
+  }
 }
 
 // ------------------------------------------------------------------------
@@ -979,8 +1456,8 @@ template <class P> __global__ void pack_kernel(const PackParams prm) {
               f32x16v even, odd;
 #pragma unroll
               for (int i = 0; i < 16; ++i) {
-                even[i] = (float)(__bf16)w[(co * cin + lo6_channel(cin, cb, 2 * i)) * 9 + tap] * sc;
-                odd[i] = (float)(__bf16)w[(co * cin + lo6_channel(cin, cb, 2 * i + 1)) * 9 + tap] * sc;
+                even[i] = (float)(__bf16)w[(co * cin + lo6_channel(cb, 2 * i)) * 9 + tap] * sc;
+                odd[i] = (float)(__bf16)w[(co * cin + lo6_channel(cb, 2 * i + 1)) * 9 + tap] * sc;
               }
               const u32x6 r = to_fp6_block(even, odd, 1.0f);
               if (piece == 0) {
@@ -1024,10 +1501,21 @@ template <class P> __global__ void pack_kernel(const PackParams prm) {
         put_elem<P>(dst, e, v);
       }
     } else {
-      const int kc_per_tap = cin / G::KSTEP;
-      const int tap = s / kc_per_tap, kc = s - tap * kc_per_tap;
+      // k-step s -> (tap, 16 or 8 input channels): tap-major, or for the pipelined kernel
+      // phase-major (a phase = all nine taps of 32 input channels)
+      int tap, cbase;
+      if constexpr (P::PIPE) {
+        constexpr int per32 = 32 / G::KSTEP;
+        const int ph = s / (9 * per32), r = s - ph * 9 * per32;
+        tap = r / per32;
+        cbase = 32 * ph + (r - tap * per32) * G::KSTEP;
+      } else {
+        const int kc_per_tap = cin / G::KSTEP;
+        tap = s / kc_per_tap;
+        cbase = (s - tap * kc_per_tap) * G::KSTEP;
+      }
       for (int e = 0; e < G::E; ++e) {
-        const int c = kc * G::KSTEP + h * G::E + e;
+        const int c = cbase + h * G::E + e;
         put_elem<P>(dst, e, w[(co * cin + c) * 9 + tap]);
       }
     }
@@ -1108,8 +1596,14 @@ template <class P> static int launch_forward(const FwdParams &fp, hipStream_t st
   hipError_t e = hipGetDevice(&dev);
   static thread_local int configured_dev = -1;
   static thread_local int cus = 0;
+  const void *kernel;
+  if constexpr (P::PIPE) {
+    kernel = reinterpret_cast<const void *>(&fused_pipe_kernel<P>);
+  } else {
+    kernel = reinterpret_cast<const void *>(&fused_forward_kernel<P>);
+  }
   if (e == hipSuccess && configured_dev != dev) {
-    e = hipFuncSetAttribute(reinterpret_cast<const void *>(&fused_forward_kernel<P>),
+    e = hipFuncSetAttribute(kernel,
                             hipFuncAttributeMaxDynamicSharedMemorySize, G::LDS_BYTES);
     int n = 0;
     if (e == hipSuccess) e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
@@ -1124,7 +1618,11 @@ template <class P> static int launch_forward(const FwdParams &fp, hipStream_t st
   }
   long long grid = cus > 0 ? cus : 256;
   if (grid > fp.total_boards) grid = fp.total_boards;
-  hipLaunchKernelGGL(fused_forward_kernel<P>, dim3((unsigned)grid), dim3(256), G::LDS_BYTES, st, fp);
+  if constexpr (P::PIPE) {
+    hipLaunchKernelGGL(fused_pipe_kernel<P>, dim3((unsigned)grid), dim3(256), G::LDS_BYTES, st, fp);
+  } else {
+    hipLaunchKernelGGL(fused_forward_kernel<P>, dim3((unsigned)grid), dim3(256), G::LDS_BYTES, st, fp);
+  }
   e = hipGetLastError();
   if (e != hipSuccess) {
     set_error("fused_forward launch failed: %s", hipGetErrorString(e));
@@ -1147,6 +1645,11 @@ int dispatch_pack(int prec, const PackParams &pp, hipStream_t st) {
 }
 
 int dispatch_forward(int prec, const FwdParams &fp, hipStream_t st) {
+#ifdef C6_ONLY_BF16F6  // (tuning builds: compile one arithmetic mode only)
+  if (prec == C6_PREC_BF16F6) return launch_forward<PrecBF16F6>(fp, st);
+  if (prec == C6_PREC_F32) return launch_forward<PrecF32>(fp, st);
+  return C6_EINVAL;
+#else
   switch (prec) {
     case C6_PREC_F32: return launch_forward<PrecF32>(fp, st);
     case C6_PREC_BF16: return launch_forward<PrecBF16>(fp, st);
@@ -1157,6 +1660,7 @@ int dispatch_forward(int prec, const FwdParams &fp, hipStream_t st) {
   }
   set_error("unknown precision mode %d", prec);
   return C6_EINVAL;
+#endif
 }
 
 size_t packed_bytes(int prec) {
