@@ -118,11 +118,26 @@ def main() -> int:
             "frac": achieved / MFMA_PEAK_TFLOPS,
             "traffic": TRAFFIC_BYTES.get(args.precision),
             "traffic_unit": "bytes per launch",
-            "kernel": "fused_forward_kernel",
+            "kernel": "fused_pipe_kernel" if args.precision in ("bf16f6", "bf16", "fp16") else "fused_forward_kernel",
             "kernel_ms": kern * 1e3,
             "flop_per_board": CONV_FLOP_PER_BOARD,
         },
     }
+    # What this card sustains on back-to-back bf16 MFMAs alone (every CU, one wave per SIMD): the
+    # published peak assumes the top shader clock, which the card's power management does not hold
+    # under a dense matrix load with ordinary operand bits.  Reported beside the roofline, which
+    # stays priced against the published peak.
+    try:
+        rnd = c6.probe_mfma_rate(60000, zero_operands=False)
+        zer = c6.probe_mfma_rate(60000, zero_operands=True)
+        out["roofline"]["sustained_mfma_only"] = {
+            "random_operands": rnd, "zero_operands": zer,
+            "frac_of_sustained": achieved / rnd["tflops"],
+            "note": "v_mfma_f32_32x32x16_bf16 back to back on all CUs; TFLOP/s over the launch (HIP events), "
+                    "mean shader clock from the cycle counter against the 100 MHz counter",
+        }
+    except c6.C6Error as exc:   # (the probe is an aid, not part of the measured path)
+        out["roofline"]["sustained_mfma_only"] = {"error": str(exc)}
 
     if not args.no_extras:
         # ---- every arithmetic mode, with its agreement with the fp32 kernel ----

@@ -4,7 +4,7 @@ Host-side mirror of the reference's operator interface for this path
 (connect6/model.py, connect6/history.py:186-303 and connect6/vector_env.py) over
 a C-ABI library of hand-written HIP kernels.
 """
-from ._lib import C6Error, build, load
+from ._lib import C6Error, build, load, probe_mfma_rate
 from .history import HistoricalCheckpoint, HistoricalPolicyEnsemble, history_dtype
 from .model import PolicyValueNet, build_model, mask_logits
 from .selfplay import (
@@ -37,6 +37,7 @@ __all__ = [
     "inverse_transform_actions",
     "load",
     "mask_logits",
+    "probe_mfma_rate",
     "sample_actions",
     "symmetry_for_phase",
     "transform_actions",

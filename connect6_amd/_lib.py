@@ -72,7 +72,41 @@ def build(verbose: bool = False) -> Path:
     if proc.returncode != 0:
         raise C6Error(f"hipcc failed ({proc.returncode}):\n" + "\n".join(other)[-4000:])
     _RESOURCES.write_text("\n".join(r.split("remark:", 1)[1].rsplit("[", 1)[0].rstrip() for r in remarks) + "\n")
+    build_probe()
     return _SO
+
+
+_PROBE_SO = _LIBDIR / "libc6_probe.so"
+
+
+def build_probe() -> Path:
+    """Compile the measurement aid ``csrc/probe/mfma_probe.hip`` (sustained bf16 MFMA rate of
+    the GPU, used by bench.py only) into ``lib/libc6_probe.so``."""
+    _LIBDIR.mkdir(exist_ok=True)
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    cmd = [hipcc, "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           "-o", str(_PROBE_SO), str(_CSRC / "probe" / "mfma_probe.hip")]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise C6Error(f"hipcc failed ({proc.returncode}):\n{proc.stderr[-4000:]}")
+    return _PROBE_SO
+
+
+def probe_mfma_rate(iters: int = 60000, zero_operands: bool = False) -> dict[str, float]:
+    """Sustained rate of back-to-back bf16 MFMAs on every CU of the current GPU (random operand
+    bits unless ``zero_operands``), and the shader clock the card holds under that load."""
+    if not _PROBE_SO.exists():
+        raise C6Error(f"{_PROBE_SO} is missing: build it with connect6_amd.build()")
+    lib = ctypes.CDLL(str(_PROBE_SO))
+    dbl = ctypes.POINTER(ctypes.c_double)
+    lib.c6_probe_mfma_rate.restype = ctypes.c_int
+    lib.c6_probe_mfma_rate.argtypes = [ctypes.c_int, ctypes.c_int, dbl, dbl, dbl]
+    tf, ghz, cyc = ctypes.c_double(), ctypes.c_double(), ctypes.c_double()
+    rc = lib.c6_probe_mfma_rate(iters, int(zero_operands), ctypes.byref(tf), ctypes.byref(ghz), ctypes.byref(cyc))
+    if rc != 0:
+        raise C6Error(f"c6_probe_mfma_rate failed with HIP error {rc}")
+    return {"tflops": tf.value, "clock_ghz": ghz.value, "cycles_per_mfma": cyc.value}
 
 
 def resource_usage(rebuild_if_missing: bool = True) -> dict[str, dict[str, int]]:

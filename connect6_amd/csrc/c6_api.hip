@@ -362,8 +362,8 @@ int c6_mask_logits(const void *logits, const uint8_t *legal, int dtype, int64_t 
     set_error("c6_mask_logits: null pointer");
     return C6_EINVAL;
   }
-  if (!aligned16(logits) || !aligned16(out) || (reinterpret_cast<uintptr_t>(legal) & 7u)) {
-    set_error("c6_mask_logits: logits/out must be 16-byte and legal 8-byte aligned");
+  if ((reinterpret_cast<uintptr_t>(logits) | reinterpret_cast<uintptr_t>(out)) & (uintptr_t)(eb - 1)) {
+    set_error("c6_mask_logits: logits/out must be aligned to their element size");
     return C6_EINVAL;
   }
   C6_REQUIRE_DEVICE("c6_mask_logits");

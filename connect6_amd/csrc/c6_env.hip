@@ -78,13 +78,19 @@ __global__ __launch_bounds__(256) void canonical_input_kernel(const int8_t *__re
                                                               long long num, int cells_arg,
                                                               float *__restrict__ out) {
   const int cells = CELLS > 0 ? CELLS : cells_arg;
-  extern __shared__ int8_t s_board[];  // kCanonGames * cells
+  extern __shared__ __attribute__((aligned(16))) int8_t s_board[];  // kCanonGames * cells, + 8 so that word reads may run past the end
   __shared__ int s_me[kCanonGames];
   __shared__ float s_last[kCanonGames];
   const long long g0 = (long long)blockIdx.x * kCanonGames;
   const int ng = (int)(num - g0 < kCanonGames ? num - g0 : kCanonGames);
   const int8_t *src = boards + g0 * cells;
-  for (int i = threadIdx.x; i < ng * cells; i += blockDim.x) s_board[i] = src[i];
+  if (ng == kCanonGames && (reinterpret_cast<uintptr_t>(src) & 7u) == 0) {
+    // eight boards = 8 * cells bytes: a whole number of 8-byte units
+    for (int i = threadIdx.x; i < cells; i += blockDim.x)
+      reinterpret_cast<v2i *>(s_board)[i] = reinterpret_cast<const v2i *>(src)[i];
+  } else {
+    for (int i = threadIdx.x; i < ng * cells; i += blockDim.x) s_board[i] = src[i];
+  }
   if ((int)threadIdx.x < ng) {
     s_me[threadIdx.x] = player[g0 + threadIdx.x];
     s_last[threadIdx.x] = stones_left[g0 + threadIdx.x] == 1 ? 1.0f : 0.0f;
@@ -100,20 +106,38 @@ __global__ __launch_bounds__(256) void canonical_input_kernel(const int8_t *__re
     return plane == 2 ? s_last[g] : ((plane == 0 ? stone == me : stone == -me) ? 1.0f : 0.0f);
   };
   if ((total & 3) == 0 && (reinterpret_cast<uintptr_t>(dst) & 15u) == 0) {
+    const unsigned *words = reinterpret_cast<const unsigned *>(s_board);
     for (int q = threadIdx.x; q < total / 4; q += blockDim.x) {
       // two divisions per four outputs: locate the first, then step through planes and games
       int g = (4 * q) / per_game, rem = 4 * q - g * per_game;
       int plane = rem / cells, cell = rem - plane * cells;
       f32x4 o;
+      if (cell + 3 < cells) {
+        // the four squares sit in one plane: fetch their bytes as one (unaligned) word and
+        // compare all four with the wanted stone at once
+        if (plane == 2) {
+          const float l = s_last[g];
+          o = f32x4{l, l, l, l};
+        } else {
+          const int a = g * cells + cell;
+          const unsigned w = __builtin_amdgcn_alignbyte(words[(a >> 2) + 1], words[a >> 2], a & 3);
+          const int me = s_me[g];
+          const unsigned want = (unsigned)((plane == 0 ? me : -me) & 0xff) * 0x01010101u;
+          const unsigned x = w ^ want;  // a zero byte = the wanted stone
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int stone = s_board[g * cells + cell], me = s_me[g];
-        o[e] = plane == 2 ? s_last[g] : ((plane == 0 ? stone == me : stone == -me) ? 1.0f : 0.0f);
-        if (++cell == cells) {
-          cell = 0;
-          if (++plane == 3) {
-            plane = 0;
-            g = g + 1 < ng ? g + 1 : g;
+          for (int e = 0; e < 4; ++e) o[e] = ((x >> (8 * e)) & 0xffu) == 0 ? 1.0f : 0.0f;
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int stone = s_board[g * cells + cell], me = s_me[g];
+          o[e] = plane == 2 ? s_last[g] : ((plane == 0 ? stone == me : stone == -me) ? 1.0f : 0.0f);
+          if (++cell == cells) {
+            cell = 0;
+            if (++plane == 3) {
+              plane = 0;
+              g = g + 1 < ng ? g + 1 : g;
+            }
           }
         }
       }
@@ -143,10 +167,10 @@ int launch_canonical_input(const int8_t *boards, const int8_t *player, const int
   const long long blocks = (num + kCanonGames - 1) / kCanonGames;
   if (n == kBoard) {
     hipLaunchKernelGGL(canonical_input_kernel<kPix>, dim3((unsigned)blocks), dim3(256),
-                       (size_t)kCanonGames * cells, st, boards, player, stones_left, num, cells, out);
+                       (size_t)kCanonGames * cells + 8, st, boards, player, stones_left, num, cells, out);
   } else {
     hipLaunchKernelGGL(canonical_input_kernel<0>, dim3((unsigned)blocks), dim3(256),
-                       (size_t)kCanonGames * cells, st, boards, player, stones_left, num, cells, out);
+                       (size_t)kCanonGames * cells + 8, st, boards, player, stones_left, num, cells, out);
   }
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {

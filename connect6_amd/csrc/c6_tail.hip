@@ -52,23 +52,25 @@ __global__ void mask2_kernel(const uint16_t *__restrict__ in, const uint8_t *__r
   }
 }
 
+// One element per thread, for operands that are only element-aligned (a row slice such as
+// logits[1:] starts 1444 bytes into its tensor).
+template <typename T>
+__global__ void mask_elem_kernel(const T *__restrict__ in, const uint8_t *__restrict__ legal,
+                                 long long n, T fill, T *__restrict__ out) {
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+    out[i] = legal[i] ? in[i] : fill;
+}
+
 // Rows of 361 elements are only 4-byte aligned, but FOUR consecutive rows span 4*361*4 =
 // 16*361 bytes and start 16-byte aligned (the tensor base is).  The kernels below therefore
 // work on groups of four boards (eight planes for the view gather) and move them with 16-byte
 // accesses; the last, partial group falls back to element accesses.
-__device__ __forceinline__ void copy_span_f32(float *dst_lds, const float *__restrict__ src,
-                                              int n_full4, int n_elems, bool vec) {
-  if (vec) {
-    for (int i = threadIdx.x; i < n_full4; i += blockDim.x)
-      reinterpret_cast<f32x4 *>(dst_lds)[i] = reinterpret_cast<const f32x4 *>(src)[i];
-  } else {
-    for (int i = threadIdx.x; i < n_elems; i += blockDim.x) dst_lds[i] = src[i];
-  }
-}
 
-// Eight boards per workgroup (two per wave): masked softmax over 361 logits and inverse-CDF
-// draw (connect6/train.py:195-213 of the reference, with the uniform supplied).  All eight
-// rows are requested up front so that enough bytes are in flight per CU to cover HBM latency.
+// Eight boards per group (two per wave): masked softmax over 361 logits and inverse-CDF draw
+// (connect6/train.py:195-213 of the reference, with the uniform supplied).  A workgroup walks
+// over groups; while it works on one group out of LDS, the next group's rows are already on
+// their way into registers, so that every CU always has reads in flight.
 constexpr int kSampleBoards = 8;
 __global__ __launch_bounds__(256) void sample_kernel(const float *__restrict__ logits,
                                                      const uint8_t *__restrict__ legal,
@@ -78,39 +80,79 @@ __global__ __launch_bounds__(256) void sample_kernel(const float *__restrict__ l
                                                      float *__restrict__ logprob) {
   __shared__ __attribute__((aligned(16))) float s_logit[kSampleBoards * kPix];
   __shared__ __attribute__((aligned(16))) uint8_t s_legal[kSampleBoards * kPix];
+  constexpr int NV = kSampleBoards * kPix / 4;       // 16-byte units of a group's logits (722)
+  constexpr int NL = kSampleBoards * kPix / 8;       // 8-byte units of its legality bytes (361)
+  constexpr int RV = (NV + 255) / 256, RL = (NL + 255) / 256;
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  const long long b0 = (long long)blockIdx.x * kSampleBoards;
-  const int nb = (int)(batch - b0 < kSampleBoards ? batch - b0 : kSampleBoards);
-  const bool full = nb == kSampleBoards;
-  copy_span_f32(s_logit, logits + (size_t)b0 * kPix, kSampleBoards * kPix / 4, nb * kPix,
-                full && (reinterpret_cast<uintptr_t>(logits) & 15u) == 0);
-  if (legal != nullptr) {
-    const uint8_t *lsrc = legal + (size_t)b0 * kPix;  // 8*361 bytes: an 8-byte aligned span
-    if (full && (reinterpret_cast<uintptr_t>(legal) & 7u) == 0) {
-      for (int i = threadIdx.x; i < kSampleBoards * kPix / 8; i += blockDim.x)
-        reinterpret_cast<v2i *>(s_legal)[i] = reinterpret_cast<const v2i *>(lsrc)[i];
-    } else {
-      for (int i = threadIdx.x; i < nb * kPix; i += blockDim.x) s_legal[i] = lsrc[i];
-    }
-  }
-  __syncthreads();
   const bool masked = legal != nullptr;
+  const bool vec = (reinterpret_cast<uintptr_t>(logits) & 15u) == 0 &&
+                   (!masked || (reinterpret_cast<uintptr_t>(legal) & 7u) == 0);
+  const long long groups = (batch + kSampleBoards - 1) / kSampleBoards;
+  f32x4 pv[RV];
+  v2i pl[RL];
+  // a full group with aligned operands travels through registers; anything else is copied
+  // element by element when its turn comes
+  auto prefetch = [&](long long g) {
+    const long long b0 = g * kSampleBoards;
+    if (g < groups && vec && batch - b0 >= kSampleBoards) {
 #pragma unroll
-  for (int r = 0; r < kSampleBoards / 4; ++r) {
-    const int bl = w + 4 * r;
-    if (bl < nb) {
-      const float *row = s_logit + bl * kPix;
-      const uint8_t *lrow = s_legal + bl * kPix;
-      int a;
-      float lp;
-      wave_sample(
-          lane, u[b0 + bl], [&](int i) { return row[i] * inv_temperature; },
-          [&](int i) { return masked ? lrow[i] != 0 : true; }, a, lp);
-      if (lane == 0) {
-        actions[b0 + bl] = a;
-        if (logprob) logprob[b0 + bl] = lp;
+      for (int r = 0; r < RV; ++r) {
+        const int i = threadIdx.x + r * 256;
+        if (i < NV) pv[r] = reinterpret_cast<const f32x4 *>(logits + (size_t)b0 * kPix)[i];
+      }
+      if (masked) {
+#pragma unroll
+        for (int r = 0; r < RL; ++r) {
+          const int i = threadIdx.x + r * 256;
+          if (i < NL) pl[r] = reinterpret_cast<const v2i *>(legal + (size_t)b0 * kPix)[i];
+        }
       }
     }
+  };
+  long long g = blockIdx.x;
+  prefetch(g);
+  for (; g < groups; g += gridDim.x) {
+    const long long b0 = g * kSampleBoards;
+    const int nb = (int)(batch - b0 < kSampleBoards ? batch - b0 : kSampleBoards);
+    if (vec && nb == kSampleBoards) {
+#pragma unroll
+      for (int r = 0; r < RV; ++r) {
+        const int i = threadIdx.x + r * 256;
+        if (i < NV) reinterpret_cast<f32x4 *>(s_logit)[i] = pv[r];
+      }
+      if (masked) {
+#pragma unroll
+        for (int r = 0; r < RL; ++r) {
+          const int i = threadIdx.x + r * 256;
+          if (i < NL) reinterpret_cast<v2i *>(s_legal)[i] = pl[r];
+        }
+      }
+    } else {
+      for (int i = threadIdx.x; i < nb * kPix; i += blockDim.x) {
+        s_logit[i] = logits[(size_t)b0 * kPix + i];
+        if (masked) s_legal[i] = legal[(size_t)b0 * kPix + i];
+      }
+    }
+    __syncthreads();
+    prefetch(g + gridDim.x);
+#pragma unroll
+    for (int r = 0; r < kSampleBoards / 4; ++r) {
+      const int bl = w + 4 * r;
+      if (bl < nb) {
+        const float *row = s_logit + bl * kPix;
+        const uint8_t *lrow = s_legal + bl * kPix;
+        int a;
+        float lp;
+        wave_sample(
+            lane, u[b0 + bl], [&](int i) { return row[i] * inv_temperature; },
+            [&](int i) { return masked ? lrow[i] != 0 : true; }, a, lp);
+        if (lane == 0) {
+          actions[b0 + bl] = a;
+          if (logprob) logprob[b0 + bl] = lp;
+        }
+      }
+    }
+    __syncthreads();  // the rows are consumed: the next group may overwrite them
   }
 }
 
@@ -258,6 +300,17 @@ static unsigned grid_for(long long work_items, int threads) {
 
 int launch_mask(const void *logits, const uint8_t *legal, int elem_bytes, long long n,
                 uint32_t fill_bits, void *out, hipStream_t st) {
+  const bool vec = ((reinterpret_cast<uintptr_t>(logits) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0 &&
+                   (reinterpret_cast<uintptr_t>(legal) & 7u) == 0;
+  if (!vec) {
+    if (elem_bytes == 4)
+      hipLaunchKernelGGL(mask_elem_kernel<uint32_t>, dim3(grid_for(n, 256)), dim3(256), 0, st,
+                         (const uint32_t *)logits, legal, n, fill_bits, (uint32_t *)out);
+    else
+      hipLaunchKernelGGL(mask_elem_kernel<uint16_t>, dim3(grid_for(n, 256)), dim3(256), 0, st,
+                         (const uint16_t *)logits, legal, n, (uint16_t)fill_bits, (uint16_t *)out);
+    return check_launch("mask_logits");
+  }
   if (elem_bytes == 4) {
     hipLaunchKernelGGL(mask4_kernel, dim3(grid_for((n >> 2) + 1, 256)), dim3(256), 0, st,
                        (const uint32_t *)logits, legal, n, fill_bits, (uint32_t *)out);
@@ -270,7 +323,9 @@ int launch_mask(const void *logits, const uint8_t *legal, int elem_bytes, long l
 
 int launch_sample(const float *logits, const uint8_t *legal, const float *u, float inv_t,
                   long long batch, long long *actions, float *logprob, hipStream_t st) {
-  hipLaunchKernelGGL(sample_kernel, dim3((unsigned)((batch + kSampleBoards - 1) / kSampleBoards)), dim3(256), 0, st, logits,
+  const long long groups = (batch + kSampleBoards - 1) / kSampleBoards;
+  const long long resident = 256LL * 8;  // eight workgroups of 256 threads fit a CU; more only queue
+  hipLaunchKernelGGL(sample_kernel, dim3((unsigned)(groups < resident ? groups : resident)), dim3(256), 0, st, logits,
                      legal, u, inv_t, batch, actions, logprob);
   return check_launch("softmax_sample");
 }

@@ -151,7 +151,9 @@ int c6_forward_generic_static(const void *x, int x_dtype, int64_t batch, int boa
 /* Out-of-place occupied-square masking of existing logits.
  * Replaces: mask_logits (connect6/model.py:123-125).
  * logits/out: device [B,361] of element type dtype; legal: device uint8 [B,361];
- * fill_bits: the fill value's bit pattern in that element type. */
+ * fill_bits: the fill value's bit pattern in that element type.  Operands that are 16-byte
+ * (legal: 8-byte) aligned take the vector kernels; anything else that is element-aligned, such
+ * as a row slice of a larger tensor, takes an element-wise kernel. */
 int c6_mask_logits(const void *logits, const uint8_t *legal, int dtype, int64_t batch,
                    uint32_t fill_bits, void *out, void *stream);
 

@@ -24,6 +24,21 @@ def test_mask_logits_bit_exact(cuda, dtype, batch):
     assert torch.equal(out.view(itype), want.view(itype))
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_mask_logits_takes_row_slices(cuda, dtype):
+    """A contiguous row slice starts 361 elements into its tensor, so it is not 16-byte aligned;
+    the reference's torch.where accepts it (connect6/model.py:123-125) and so does this."""
+    logits = torch.randn(9, 361, generator=torch.Generator().manual_seed(3)).to(dtype)
+    _, legal = gen_boards(9, 300, 4)
+    lg, ll = logits.to(cuda), legal.to(cuda)
+    for lo in (1, 2, 3):
+        out = c6.mask_logits(lg[lo:], ll[lo:]).cpu()
+        want = R.mask_logits(logits[lo:], legal[lo:])
+        itype = torch.int32 if dtype == torch.float32 else torch.int16
+        assert torch.equal(out.view(itype), want.view(itype))
+
+
 def _check_samples(actions, logprob, logits, legal, u, temperature):
     a_ref, lp_ref = R.sample_inverse_cdf(logits, legal, u, temperature)
     actions, logprob = actions.cpu(), logprob.cpu()
