@@ -164,7 +164,13 @@ template <class P> struct Geo {
   // pipelined kernel: a copy of the weight set's fp32 tail (biases, head weights), so that no
   // layer starts, and the heads do not run, behind the latency of global loads
   static constexpr int TAIL_LDS_OFF = RED_OFF + 64;
-  static constexpr int LDS_BYTES = TAIL_LDS_OFF + (P::PIPE ? (kBiasTotal + 2 * kHeadC + 4) * 4 : 0);
+  // ... and the next board's input as the loads deliver it, one dword per element: words
+  // [0, 1083) the three planes, words 1084 / 1085 side to move / stones left (board-state input),
+  // words [1088, 1088 + 361) the legality bytes or the int8 stones.  The loads write LDS
+  // directly, so the input never sits in registers (or, under register pressure, in scratch).
+  static constexpr int NEXT_IN_OFF = TAIL_LDS_OFF + (kBiasTotal + 2 * kHeadC + 4) * 4;
+  static constexpr int NEXT_IN_AUX = 1084, NEXT_IN_BYTES_AT = 1088;
+  static constexpr int LDS_BYTES = P::PIPE ? NEXT_IN_OFF + (NEXT_IN_BYTES_AT + 384) * 4 : TAIL_LDS_OFF;
 
   static constexpr int layer_steps(int l) { return l == 0 ? STEPS1 : 9 * kCinArr[l] / KSTEP; }
   static constexpr int layer_frags(int l) { return layer_steps(l) * (kCoutArr[l] / 32); }

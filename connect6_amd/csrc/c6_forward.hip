@@ -1153,41 +1153,78 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
   auto packed_of = [&](long long b) {
     return prm.packed + (size_t)((unsigned)b / per_group) * prm.packed_stride;
   };
-  // input of one board: each thread owns pixels tid, tid + THREADS, ... (three planes + occupancy)
-  float xin[ROUNDS][3];
-  unsigned char occin[ROUNDS];
-  auto fetch_board = [&](long long b) {
+  // Input of one board, asked for a whole board ahead: loads that write LDS directly, 64
+  // consecutive elements per instruction (lane l's element lands in word l behind the
+  // instruction's LDS base).  Wave w issues chunks w, w + 4, ...
+  typedef const __attribute__((address_space(1))) void *GPtr;
+  typedef __attribute__((address_space(3))) void *LPtr;
+  auto board_row = [&](long long b) {  // board-state input: which row of the state tensors
+    long long src = prm.index ? prm.index[b] : b;
+    return src < 0 ? 0 : (src >= prm.num_states ? prm.num_states - 1 : src);
+  };
+  auto issue_fetch = [&](long long b) {
+    unsigned char *dst = smem + G::NEXT_IN_OFF;
     if (prm.x_dtype == C6_DT_BOARD_I8) {
-      // environment state in, network planes out (connect6/vector_env.py:196-218 of the
-      // reference), seen through D4 view prm.view (connect6/train.py:222-230)
-      long long src = prm.index ? prm.index[b] : b;
-      src = src < 0 ? 0 : (src >= prm.num_states ? prm.num_states - 1 : src);
+      // environment state (connect6/vector_env.py:196-218 of the reference), seen through D4
+      // view prm.view (connect6/train.py:222-230): the stones, the side to move, stones left
+      const long long src = board_row(b);
       const int8_t *board = reinterpret_cast<const int8_t *>(prm.x) + (size_t)src * kPix;
-      const int me = prm.player[src];
-      const float last = prm.stones_left[src] == 1 ? 1.0f : 0.0f;
-#pragma unroll
-      for (int r = 0; r < ROUNDS; ++r) {
-        const int p = tid + r * THREADS;
-        if (p < kPix) {
-          const int stone = board[prm.view ? d4_from_view(p, prm.view) : p];
-          xin[r][0] = stone == me ? 1.0f : 0.0f;
-          xin[r][1] = stone == -me ? 1.0f : 0.0f;
-          xin[r][2] = last;
-          occin[r] = 0;
-        }
+      for (int i = wave; i < (kPix + 63) / 64; i += NWAVES) {
+        const int p = i * 64 + lane;
+        if (p < kPix)
+          __builtin_amdgcn_global_load_lds((GPtr)(board + (prm.view ? d4_from_view(p, prm.view) : p)),
+                                           (LPtr)(dst + (G::NEXT_IN_BYTES_AT + i * 64) * 4), 1, 0, 0);
       }
+      if (wave == 0 && lane < 2)
+        __builtin_amdgcn_global_load_lds((GPtr)((lane == 0 ? prm.player : prm.stones_left) + src),
+                                         (LPtr)(dst + G::NEXT_IN_AUX * 4), 1, 0, 0);
       return;
     }
-#pragma unroll
-    for (int r = 0; r < ROUNDS; ++r) {
-      const int p = tid + r * THREADS;
-      if (p < kPix) {
-#pragma unroll
-        for (int ch = 0; ch < 3; ++ch)
-          xin[r][ch] = load_x(prm.x, prm.x_dtype, ((size_t)b * 3 + ch) * kPix + p);
-        occin[r] = prm.mask_mode == C6_MASK_LEGAL ? (prm.legal[(size_t)b * kPix + p] == 0) : 0;
+    constexpr int NE = 3 * kPix;
+    if (prm.x_dtype == C6_DT_F32) {
+      const float *xf = reinterpret_cast<const float *>(prm.x) + (size_t)b * NE;
+      for (int i = wave; i < (NE + 63) / 64; i += NWAVES) {
+        const int e = i * 64 + lane;
+        if (e < NE) __builtin_amdgcn_global_load_lds((GPtr)(xf + e), (LPtr)(dst + i * 256), 4, 0, 0);
+      }
+    } else {
+      const unsigned short *xh = reinterpret_cast<const unsigned short *>(prm.x) + (size_t)b * NE;
+      for (int i = wave; i < (NE + 63) / 64; i += NWAVES) {
+        const int e = i * 64 + lane;
+        if (e < NE) __builtin_amdgcn_global_load_lds((GPtr)(xh + e), (LPtr)(dst + i * 256), 2, 0, 0);
       }
     }
+    if (prm.mask_mode == C6_MASK_LEGAL) {
+      const uint8_t *lg = prm.legal + (size_t)b * kPix;
+      for (int i = wave; i < (kPix + 63) / 64; i += NWAVES) {
+        const int p = i * 64 + lane;
+        if (p < kPix)
+          __builtin_amdgcn_global_load_lds((GPtr)(lg + p), (LPtr)(dst + (G::NEXT_IN_BYTES_AT + i * 64) * 4), 1, 0, 0);
+      }
+    }
+  };
+  // what arrived for square p: the three planes and the occupancy flag
+  auto staged_input = [&](int p, float (&v)[3], unsigned &o) {
+    const unsigned *raw = reinterpret_cast<const unsigned *>(smem + G::NEXT_IN_OFF);
+    const unsigned aux = raw[G::NEXT_IN_BYTES_AT + p] & 0xffu;
+    if (prm.x_dtype == C6_DT_BOARD_I8) {
+      const int stone = (int8_t)aux, me = (int8_t)(raw[G::NEXT_IN_AUX] & 0xffu);
+      v[0] = stone == me ? 1.0f : 0.0f;
+      v[1] = stone == -me ? 1.0f : 0.0f;
+      v[2] = (raw[G::NEXT_IN_AUX + 1] & 0xffu) == 1 ? 1.0f : 0.0f;
+    } else {
+#pragma unroll
+      for (int ch = 0; ch < 3; ++ch) {
+        const unsigned w = raw[ch * kPix + p];
+        const float as_bf16 = __builtin_bit_cast(float, w << 16);
+        const float as_f16 = (float)__builtin_bit_cast(_Float16, (unsigned short)w);
+        v[ch] = prm.x_dtype == C6_DT_F32 ? __builtin_bit_cast(float, w)
+                                          : (prm.x_dtype == C6_DT_BF16 ? as_bf16 : as_f16);
+      }
+    }
+    o = 0;
+    if (prm.mask_mode == C6_MASK_LEGAL) o = aux == 0;
+    if (prm.mask_mode == C6_MASK_INPUT) o = (v[0] != 0.0f) || (v[1] != 0.0f);
   };
 
   // Each workgroup takes one contiguous run of boards, and the runs are dealt out so that the
@@ -1203,7 +1240,7 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
   [[maybe_unused]] const long long b_first = b;
   v4i r1[L1Pipe<P>::D][1];
   preload_ring<L1Pipe<P>::D, 1>(r1, layer_weights<P, 0>(packed_of(b), lane));
-  fetch_board(b);
+  issue_fetch(b);
 
   for (; b < b_end; ++b) {
     int tidv = tid;  // opaque per board: keeps per-thread staging addresses out of long-lived registers
@@ -1235,8 +1272,10 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
 #else
     const bool trace_on = false;
 #endif
-    __syncthreads();  // previous board fully written out; LDS is free
+    __builtin_amdgcn_s_waitcnt(0);  // this wave's share of the board's input has landed in LDS
+    __syncthreads();  // ... and everybody's; previous board fully written out; LDS is free
     C6_MARK(0);
+    const long long bn = b + 1;
     // ---- stage the input: zero the shifted copies, then scatter the board ----
     {
       const v4i z = {0, 0, 0, 0};
@@ -1249,16 +1288,18 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
       const int p = tidv + r * THREADS;
       if (p < kPix) {
         const int row = p / kBoard, c = p - row * kBoard;
-        unsigned char o = occin[r];
-        if (prm.mask_mode == C6_MASK_INPUT) o = (xin[r][0] != 0.0f) || (xin[r][1] != 0.0f);
-        occ[p] = o;
+        float v[3];
+        unsigned o;
+        staged_input(p, v, o);
+        occ[p] = (unsigned char)o;
 #pragma unroll
         for (int ch = 0; ch < 3; ++ch) {
           const int hrow = (row + kK1 / 2) * 3 + ch;
+          const unsigned short v16 = bits16<P>(v[ch]);
 #pragma unroll
           for (int s = 0; s < G::E; ++s) {
             const int a = s * G::COPY_BYTES + (hrow * kL1RowPitch + (c + kK1 / 2 - s)) * G::EB;
-            *reinterpret_cast<unsigned short *>(smem + a) = bits16<P>(xin[r][ch]);
+            *reinterpret_cast<unsigned short *>(smem + a) = v16;
           }
         }
       }
@@ -1269,8 +1310,6 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
         if (tidv + r * THREADS < TAILN)
           reinterpret_cast<float *>(smem + G::TAIL_LDS_OFF)[tidv + r * THREADS] = tailv[r];
     }
-    const long long bn = b + 1;
-    if (bn < b_end) fetch_board(bn);  // lands while this board is computed
     __syncthreads();
     C6_MARK(1);
 
@@ -1318,6 +1357,10 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
       asm volatile("" : "+v"(hb));  // (one address register for all head weights)
       const float *pwg = reinterpret_cast<const float *>(smem + hb);
       const float *tl = pwg - 4 * h - kBiasTotal;
+      // The next board's input is asked for here: the counter of loads in flight is served in
+      // order, so in front of a K-loop these loads from HBM would hold up its weight fragments,
+      // while the heads wait for no load at all.
+      if (bn < b_end) issue_fetch(bn);
       if (bn < b_end) preload_ring<L1Pipe<P>::D, 1>(r1, layer_weights<P, 0>(packed_of(bn), lane));
       float pol[3] = {0.0f, 0.0f, 0.0f};
       float vsum = 0.0f;
