@@ -61,56 +61,92 @@ __device__ __forceinline__ float wave_inclusive_sum(float v) {
 }
 
 // Masked softmax + inverse-CDF draw over 361 entries by ONE wave.
-// z(i) must return the tempered logit of entry i, ok(i) its legality.
-// action = first i with running sum of exp(z - max) > u * total, clamped to
-// the last legal entry; logp = z[a] - max - log(total).
+// z(i) must return the logit of entry i, ok(i) its legality; inv_t = 1 / temperature.
+// action = first i with running sum of exp(z/T - max) > u * total, clamped to the last legal
+// entry; logp = z[a]/T - max - log(total).
+// The kernels that call this are bound by its VALU instructions, so it is written to need few:
+// logits are carried in units of log2 (one multiply per entry, a bare v_exp_f32 each), an illegal
+// entry is -inf and exponentiates to 0 by itself, the lane that holds the draw is found with a
+// ballot, and the last legal entry is only looked for when no running sum exceeds the target
+// (u * total rounding up to the total).
 template <class FZ, class FOK>
-__device__ __forceinline__ void wave_sample(int lane, float u, FZ z, FOK ok, int &action,
+__device__ __forceinline__ void wave_sample(int lane, float u, float inv_t, FZ z, FOK ok, int &action,
                                             float &logp) {
   constexpr int PER = 6;  // 64 lanes x 6 = 384 >= 361
+  constexpr float kLog2e = 1.4426950408889634f, kLn2 = 0.6931471805599453f;
+  const float s2 = inv_t * kLog2e;
   float zz[PER];
-  bool lg[PER];
   float m = -INFINITY;
-  int lastlegal = -1;
 #pragma unroll
   for (int e = 0; e < PER; ++e) {
     const int i = lane * PER + e;
-    lg[e] = (i < kPix) && ok(i);
-    zz[e] = lg[e] ? z(i) : -INFINITY;
+    zz[e] = ((i < kPix) && ok(i)) ? z(i) * s2 : -INFINITY;
     m = fmaxf(m, zz[e]);
-    if (lg[e]) lastlegal = i;
   }
   m = wave_max(m);
-  lastlegal = wave_max_i(lastlegal);
-  float ex[PER];
+  const float mc = fmaxf(m, -3.0e38f);  // (no legal entry at all: exp2(-inf - mc) stays 0, not NaN)
+  float run[PER];
   float local = 0.0f;
 #pragma unroll
   for (int e = 0; e < PER; ++e) {
-    ex[e] = lg[e] ? __expf(zz[e] - m) : 0.0f;
-    local += ex[e];
+    local += __builtin_amdgcn_exp2f(zz[e] - mc);
+    run[e] = local;  // running sum inside the lane
   }
-  // inclusive scan of lane sums
   const float incl = wave_inclusive_sum(local);
   const float total = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, incl), 63));
   const float target = u * total;
-  float run = incl - local;
-  int first = 1 << 30;
+  // the first lane whose inclusive sum exceeds the target holds the draw
+  const unsigned long long over = __builtin_amdgcn_ballot_w64(incl > target);
+  int first;
+  if (over != 0) {
+    const int owner = __builtin_ctzll(over);
+    const float before = incl - local;
+    int cnt = 0;  // entries of this lane whose running sum does not exceed the target yet
 #pragma unroll
-  for (int e = 0; e < PER; ++e) {
-    run += ex[e];
-    if (lg[e] && run > target && first == (1 << 30)) first = lane * PER + e;
+    for (int e = 0; e < PER; ++e) cnt += (before + run[e] > target) ? 0 : 1;
+    cnt = cnt < PER ? cnt : PER - 1;  // ((incl - local) + local may round below incl)
+    float zsel = zz[PER - 1];
+#pragma unroll
+    for (int e = PER - 2; e >= 0; --e) zsel = cnt == e ? zz[e] : zsel;
+    first = owner * PER + __builtin_amdgcn_readlane(cnt, owner);
+    float za = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, zsel), owner));
+    if (za == -INFINITY) {
+      // Rounding put the draw on an illegal entry next to the step it belongs to (the lanes'
+      // sums disagree in the last bit): take the nearest legal entry below, else above.
+      int below = -1, above = 1 << 30;
+#pragma unroll
+      for (int e = 0; e < PER; ++e) {
+        const int i = lane * PER + e;
+        if (zz[e] != -INFINITY) {
+          if (i <= first) below = i;
+          if (i > first && above == (1 << 30)) above = i;
+        }
+      }
+      below = wave_max_i(below);
+      above = wave_min_i(above);
+      first = below >= 0 ? below : above;
+      float zf = -INFINITY;
+#pragma unroll
+      for (int e = 0; e < PER; ++e)
+        if (lane * PER + e == first) zf = zz[e];
+      za = wave_max(zf);
+    }
+    logp = (za - m) * kLn2 - __logf(total);
+  } else {
+    int lastlegal = -1;
+#pragma unroll
+    for (int e = 0; e < PER; ++e)
+      if (zz[e] != -INFINITY) lastlegal = lane * PER + e;
+    lastlegal = wave_max_i(lastlegal);
+    first = lastlegal < 0 ? 0 : lastlegal;  // no legal square at all: defined but meaningless
+    float za = -INFINITY;
+#pragma unroll
+    for (int e = 0; e < PER; ++e)
+      if (lane * PER + e == first) za = zz[e];
+    za = wave_max(za);
+    logp = (za - m) * kLn2 - __logf(total);
   }
-  first = wave_min_i(first);
-  if (first == (1 << 30)) first = lastlegal;
-  if (first < 0) first = 0;  // no legal square at all: defined but meaningless
   action = first;
-  // fetch z[action] from the lane that holds it
-  float za = 0.0f;
-#pragma unroll
-  for (int e = 0; e < PER; ++e)
-    if (lane * PER + e == first) za = zz[e];
-  za = wave_max(lane == first / PER ? za : -INFINITY);
-  logp = za - m - __logf(total);
 }
 
 

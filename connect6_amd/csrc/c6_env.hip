@@ -107,10 +107,18 @@ __global__ __launch_bounds__(256) void canonical_input_kernel(const int8_t *__re
   };
   if ((total & 3) == 0 && (reinterpret_cast<uintptr_t>(dst) & 15u) == 0) {
     const unsigned *words = reinterpret_cast<const unsigned *>(s_board);
-    for (int q = threadIdx.x; q < total / 4; q += blockDim.x) {
-      // two divisions per four outputs: locate the first, then step through planes and games
-      int g = (4 * q) / per_game, rem = 4 * q - g * per_game;
-      int plane = rem / cells, cell = rem - plane * cells;
+    // (game, offset inside the game) of the thread's first output, then stepped by 4 * blockDim
+    // per iteration: no division in the loop
+    int g = (4 * (int)threadIdx.x) / per_game, rem = 4 * (int)threadIdx.x - g * per_game;
+    const int step = 4 * (int)blockDim.x, step_g = step / per_game, step_rem = step - step_g * per_game;
+    for (int q = threadIdx.x; q < total / 4; q += blockDim.x, g += step_g, rem += step_rem) {
+      if (rem >= per_game) {
+        rem -= per_game;
+        ++g;
+      }
+      int plane = rem >= 2 * cells ? 2 : (rem >= cells ? 1 : 0);
+      int cell = rem - plane * cells;
+      const int g_first = g;
       f32x4 o;
       if (cell + 3 < cells) {
         // the four squares sit in one plane: fetch their bytes as one (unaligned) word and
@@ -128,15 +136,16 @@ __global__ __launch_bounds__(256) void canonical_input_kernel(const int8_t *__re
           for (int e = 0; e < 4; ++e) o[e] = ((x >> (8 * e)) & 0xffu) == 0 ? 1.0f : 0.0f;
         }
       } else {
+        int gg = g_first;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          const int stone = s_board[g * cells + cell], me = s_me[g];
-          o[e] = plane == 2 ? s_last[g] : ((plane == 0 ? stone == me : stone == -me) ? 1.0f : 0.0f);
+          const int stone = s_board[gg * cells + cell], me = s_me[gg];
+          o[e] = plane == 2 ? s_last[gg] : ((plane == 0 ? stone == me : stone == -me) ? 1.0f : 0.0f);
           if (++cell == cells) {
             cell = 0;
             if (++plane == 3) {
               plane = 0;
-              g = g + 1 < ng ? g + 1 : g;
+              gg = gg + 1 < ng ? gg + 1 : gg;
             }
           }
         }

@@ -1418,7 +1418,7 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
       int a;
       float lp;
       wave_sample(
-          lane, prm.u[b], [&](int i) { return lgt[i] * it; }, [&](int i) { return occ[i] == 0; },
+          lane, prm.u[b], it, [&](int i) { return lgt[i]; }, [&](int i) { return occ[i] == 0; },
           a, lp);
       if (lane == 0) {
         prm.actions[b] = a;
@@ -1678,7 +1678,7 @@ __global__ __launch_bounds__(256) void fused_forward_kernel(const FwdParams prm)
       int a;
       float lp;
       wave_sample(
-          lane, prm.u[b], [&](int i) { return lgt[i] * it; }, [&](int i) { return occ[i] == 0; },
+          lane, prm.u[b], it, [&](int i) { return lgt[i]; }, [&](int i) { return occ[i] == 0; },
           a, lp);
       if (lane == 0) {
         prm.actions[b] = a;

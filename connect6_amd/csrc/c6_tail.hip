@@ -144,7 +144,7 @@ __global__ __launch_bounds__(256) void sample_kernel(const float *__restrict__ l
         int a;
         float lp;
         wave_sample(
-            lane, u[b0 + bl], [&](int i) { return row[i] * inv_temperature; },
+            lane, u[b0 + bl], inv_temperature, [&](int i) { return row[i]; },
             [&](int i) { return masked ? lrow[i] != 0 : true; }, a, lp);
         if (lane == 0) {
           actions[b0 + bl] = a;
