@@ -709,29 +709,23 @@ __device__ __forceinline__ void mid_layer(
 //
 // With one wave per SIMD nothing runs beside a wave's own instruction stream, and the SiLU
 // epilogue of a layer (two transcendentals per element) used to run with the matrix pipe idle.
-// VALU work issued between the MFMAs of a K-loop is nearly free (a full SiLU per MFMA lengthens
-// a 33-cycle MFMA slot by 7 cycles), so the epilogue of layer L is issued from inside the K-loop
-// of layer L+1: that loop is ordered phase-major, a phase being all nine taps of 32 input
-// channels = one cout tile of layer L.  Only cout tile 0 of layer L is converted in the open;
-// phase p of layer L+1 then carries the conversion of tile p+1, with a barrier between phases.
-// The accumulators of layer L therefore stay live next to those of layer L+1.
+// A few VALU instructions issued behind each MFMA of a K-loop cost little (a lone wave issues
+// one instruction per ~5 cycles and an MFMA occupies the matrix pipe for 32), so the epilogues
+// are issued from inside K-loops.  A 3x3 layer's K is ordered phase-major, a phase being all nine
+// taps of 32 input channels = one cout tile of the layer before.  Phase p carries the epilogue of
+// tile p+1 of the layer before (whose accumulators stay live next to this layer's), and the last
+// phase runs cout tile 0 first and carries that tile's own epilogue behind the other tiles' MFMAs
+// (pipe_layer).  Only single-tile layers convert anything with the matrix pipe idle.
 // ------------------------------------------------------------------------
 constexpr int kPhaseSteps = 18;   // k-steps of one phase: 9 taps x 2 k-steps of 16 channels
 
-// even K slots of a 192-bit fp6 block, as three repeating dword masks (slot s = bits [6s, 6s+6))
-__host__ __device__ constexpr unsigned fp6_even_mask(int dword) {
-  unsigned m = 0;
-  for (int b = 0; b < 32; ++b)
-    if ((32 * dword + b) % 12 < 6) m |= 1u << b;
-  return m;
-}
-
 // The epilogue of one cout tile (SiLU, bf16 store, low-order fp6 blocks) as a list of atoms --
 // single instructions or short groups -- that a compile-time schedule deals out over the MFMA
-// slots of the next layer's K-loop.  A wave issues one instruction every ~4 cycles and an MFMA
-// occupies the matrix pipe for 32, so about six other instructions fit behind it
-// (transcendentals count double, and the K-loop's own LDS reads and weight loads need their
-// share): the schedule gives every slot the same small budget of VALU cycles.
+// slots of a K-loop segment.  A lone wave issues one instruction every ~5 cycles and an MFMA
+// occupies the matrix pipe for 32, so about six instructions fit into a slot, the MFMA, the
+// K-loop's own LDS reads, weight loads and waits included; measured, about two VALU instructions
+// per slot ride for free and every further one costs its full issue time.  The schedule
+// therefore spreads the atoms evenly: every slot gets the same small budget.
 // The lane's elements (3 pixel tiles x its channels of the cout tile) stream through a software
 // pipeline, so that consecutive atoms never depend on each other:
 //   step s:  exp2 of element s | 1 + . of element s-1 | rcp of element s-2 | x * . of element s-3

@@ -394,3 +394,29 @@ def test_c_abi_from_a_plain_cpp_program(cuda):
     print(proc.stdout)
     assert proc.returncode == 0, proc.stdout + proc.stderr
     assert "all checks passed" in proc.stdout
+
+
+def test_sustained_mfma_probe_reports_a_plausible_rate(cuda):
+    """bench.py's reference point: bf16 MFMAs alone, every CU.  All-zero operands draw little
+    power and run near the top clock; ordinary operand bits must not be faster than that."""
+    rnd = c6.probe_mfma_rate(20000, zero_operands=False)
+    zer = c6.probe_mfma_rate(20000, zero_operands=True)
+    for r in (rnd, zer):
+        assert 31.5 <= r["cycles_per_mfma"] <= 36.0          # one 32x32x16 MFMA = 32 cycles of the matrix pipe
+        assert 0.8 <= r["clock_ghz"] <= 2.6
+        assert 500.0 <= r["tflops"] <= 2600.0                 # never above the published 2.5 PFLOP/s (+ timer slack)
+    assert rnd["tflops"] <= zer["tflops"] * 1.05
+
+
+def test_phase_profile_runs_when_the_traced_library_is_built(cuda):
+    import subprocess
+    import sys
+
+    from connect6_amd import profiling
+
+    if not profiling.TRACE_SO.exists():
+        pytest.skip("python -m connect6_amd.profiling --build was not run")
+    out = subprocess.run([sys.executable, "-m", "connect6_amd.profiling", "bf16f6"], capture_output=True,
+                         text=True, timeout=280)
+    assert out.returncode == 0, out.stderr[-2000:]
+    assert "one board =" in out.stdout and "conv8 low-order pass" in out.stdout

@@ -308,3 +308,12 @@ def test_bench_refuses_more_than_one_gpu():
     proc = subprocess.run([sys.executable, str(ROOT / "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert proc.returncode != 0
     assert "one GPU" in proc.stderr and proc.stdout.strip() == ""
+
+
+def test_probe_library_loads_and_exports_its_symbol():
+    # the measurement aid bench.py uses (sustained bf16 MFMA rate); no compute without a GPU
+    import ctypes
+
+    assert _lib._PROBE_SO.exists(), "run connect6_amd.build()"
+    probe = ctypes.CDLL(str(_lib._PROBE_SO))
+    assert hasattr(probe, "c6_probe_mfma_rate")
