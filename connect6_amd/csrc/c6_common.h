@@ -192,7 +192,21 @@ template <class P> struct Geo {
     return s;
   }
   static constexpr int LO_FRAGS = P::LO8 ? (lo_frag_offset(8) - HI_FRAGS) + kLoRing * 3 * 2 : 0;
-  static constexpr int TOTAL_FRAGS = HI_FRAGS + LO_FRAGS;
+  // Pipelined kernel, first layer on a board whose third plane is one constant c (what the
+  // reference feeds it: the "last stone of the turn" flag broadcast over the board,
+  // connect6/vector_env.py:211-217): that plane's contribution is c * (sum of its weights
+  // inside the board, seen from the output square) -- a per-square table, added with the bias --
+  // and K shrinks to the other two planes, one per lane half: 23 kernel rows x 3 fragments of
+  // 8 columns = 69 k-steps instead of 105.  A second copy of the first layer's weights in that
+  // order follows the low-order copies, then the table, laid out as the lanes hold it: fragment
+  // ((wave * 3 + pixel tile) * 4 + q) = 64 lanes x four fp32 (channels 8 q + 4 h .. + 3 of the
+  // lane's square), one coalesced 16-byte load per lane each.
+  static constexpr int FAST1_STEPS = kK1 * CPR;
+  static constexpr int FAST1_OFF = HI_FRAGS + LO_FRAGS;  // in 1 KiB fragments
+  static constexpr int PLANE2_FRAG_OFF = FAST1_OFF + FAST1_STEPS + 8;  // (8 zero fragments: over-read)
+  static constexpr int PLANE2_FRAGS = kWaves * 3 * 4;
+  static constexpr int FAST1_FRAGS = (P::PIPE && EB == 2) ? FAST1_STEPS + 8 + PLANE2_FRAGS : 0;
+  static constexpr int TOTAL_FRAGS = HI_FRAGS + LO_FRAGS + FAST1_FRAGS;
   static constexpr size_t TAIL_OFF = (size_t)TOTAL_FRAGS * 1024;  // fp32 tail: biases, heads
   // tail words: bias[544] polw[96] valw[96] polb valb pad pad, then 8 ints sw[layer]
   static constexpr int TAIL_SW = kBiasTotal + 2 * kHeadC + 4;

@@ -338,6 +338,39 @@ __device__ __forceinline__ void conv1_pass(const unsigned char *smem, const WFra
   }
 }
 
+// First layer when the third input plane is constant: K = (ky, kx24) of planes 0 and 1, plane h
+// in lane half h (Geo::FAST1_*).  l1fast[j]: as l1base, for halo row 3 r + h.
+// `ring`: a FIFO over the fragment stream (fragment s in slot s % D), filled with its first D.
+template <class P>
+__device__ __forceinline__ void conv1_fast_pass(const unsigned char *smem, const WFrags &wl,
+                                                v4i (&ring)[L1Pipe<P>::D][1], const int (&l1fast)[3],
+                                                f32x16 (&acc)[1][3]) {
+  using G = Geo<P>;
+  constexpr int CPR = G::CPR, D = L1Pipe<P>::D, QN = kAhead + 1, S = G::FAST1_STEPS;
+  constexpr int ROWB = kL1RowPitch * G::EB;
+  static_assert(S % QN == 0, "fragment queue must line up");
+  auto frag = [&](int j, int s) {  // kernel row s / CPR is three halo rows further down
+    return *reinterpret_cast<const v4i *>(smem + l1fast[j] + (s / CPR) * 3 * ROWB + (s % CPR) * 16);
+  };
+  v4i bq[QN][3];
+#pragma unroll
+  for (int a = 0; a < kAhead; ++a)
+#pragma unroll
+    for (int j = 0; j < 3; ++j) bq[a][j] = frag(j, a);
+  static_for<0, S>([&](auto sc) __attribute__((always_inline)) {
+    constexpr int s = decltype(sc)::value;
+    if constexpr (s + kAhead < S) {
+#pragma unroll
+      for (int j = 0; j < 3; ++j) bq[(s + kAhead) % QN][j] = frag(j, s + kAhead);
+    }
+#pragma unroll
+    for (int j = 0; j < 3; ++j) mma<P>(ring[s % D][0], bq[s % QN][j], acc[0][j]);
+    ring[s % D][0] = wl[s + D];  // (the tail over-reads the zero fragments behind the stream)
+    interleave_step<3, 3, 1>();
+    __builtin_amdgcn_sched_barrier(0);
+  });
+}
+
 // ------------------------------------------------------------------------
 // 3x3 layers: K = (tap, cin), cin fastest; taps are constant position offsets
 // ------------------------------------------------------------------------
@@ -1220,6 +1253,12 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
     if (prm.mask_mode == C6_MASK_LEGAL) o = aux == 0;
     if (prm.mask_mode == C6_MASK_INPUT) o = (v[0] != 0.0f) || (v[1] != 0.0f);
   };
+  // the third plane's value at square 0, and whether square p holds another one
+  auto plane2_differs = [&](int p) {
+    const unsigned *raw = reinterpret_cast<const unsigned *>(smem + G::NEXT_IN_OFF);
+    return prm.x_dtype != C6_DT_BOARD_I8 && raw[2 * kPix + p] != raw[2 * kPix];
+  };
+  auto fast1_weights = [&](long long b) { return packed_frags<P>(packed_of(b), lane, G::FAST1_OFF); };
 
   // Each workgroup takes one contiguous run of boards, and the runs are dealt out so that the
   // workgroups of one XCD (workgroup i runs on XCD i % 8) cover one contiguous eighth of the
@@ -1233,7 +1272,9 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
   if (b >= b_end) return;
   [[maybe_unused]] const long long b_first = b;
   v4i r1[L1Pipe<P>::D][1];
-  preload_ring<L1Pipe<P>::D, 1>(r1, layer_weights<P, 0>(packed_of(b), lane));
+  // (the first layer's weight ring is filled, a board ahead, with the stream for a constant
+  // third plane; a board that has none refills it)
+  preload_ring<L1Pipe<P>::D, 1>(r1, fast1_weights(b));
   issue_fetch(b);
 
   for (; b < b_end; ++b) {
@@ -1270,13 +1311,34 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
     __syncthreads();  // ... and everybody's; previous board fully written out; LDS is free
     C6_MARK(0);
     const long long bn = b + 1;
+    // The third plane's share of the first layer, should the plane turn out constant: the
+    // per-square sums of its weights (register i of pixel tile j = channel 8 (i / 4) + 4 h + i % 4),
+    // asked for now so that the loads are long back when the K-loop starts; there they are
+    // multiplied by the plane's value and joined by the bias.
+    f32x16 a0[1][3];
+    {
+      // (the wave number through a scalar register: the loads take the fragment offset from one)
+      const WFrags tb = packed_frags<P>(packed, lane, G::PLANE2_FRAG_OFF + __builtin_amdgcn_readfirstlane(wave) * 12);
+#pragma unroll
+      for (int j = 0; j < 3; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const f32x4 t4 = __builtin_bit_cast(f32x4, tb[j * 4 + q]);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) a0[0][j][4 * q + e] = t4[e];
+        }
+      __builtin_amdgcn_sched_barrier(0);  // (issue here)
+    }
     // ---- stage the input: zero the shifted copies, then scatter the board ----
+    int *plane2_flag = reinterpret_cast<int *>(red) + 8;  // set by any thread that sees the third plane vary
+    if (tid == 0) *plane2_flag = 0;
     {
       const v4i z = {0, 0, 0, 0};
       for (int i = tidv * 16; i < G::COPIES_BYTES; i += THREADS * 16)
         *reinterpret_cast<v4i *>(smem + i) = z;
     }
     __syncthreads();
+    bool varies = false;
 #pragma unroll
     for (int r = 0; r < ROUNDS; ++r) {
       const int p = tidv + r * THREADS;
@@ -1285,6 +1347,7 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
         float v[3];
         unsigned o;
         staged_input(p, v, o);
+        varies |= plane2_differs(p);
         occ[p] = (unsigned char)o;
 #pragma unroll
         for (int ch = 0; ch < 3; ++ch) {
@@ -1304,19 +1367,37 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
         if (tidv + r * THREADS < TAILN)
           reinterpret_cast<float *>(smem + G::TAIL_LDS_OFF)[tidv + r * THREADS] = tailv[r];
     }
+    if (varies) *plane2_flag = 1;
     __syncthreads();
+    const bool plane2_varies = *plane2_flag != 0;
     C6_MARK(1);
 
     v4i r2[kRing], r3[kRing * 2], r6[kRing * 3];  // weight rings of layers 2, 3-5, 6-8
-    f32x16 a0[1][3], a1[1][3];
+    f32x16 a1[1][3];
     // ---- layer 1 ----
     {
       f32x16 b0[1];
       load_bias_tiles_lds(b0, smem, tail_lds, bias_offset(0), h);
+      if (!plane2_varies) {
+        float v2[3];
+        unsigned o2;
+        staged_input(0, v2, o2);
+        const float c2 = v2[2];
 #pragma unroll
-      for (int j = 0; j < 3; ++j) a0[0][j] = b0[0];
+        for (int j = 0; j < 3; ++j)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) a0[0][j][i] = fmaf(c2, a0[0][j][i], b0[0][i]);
+        int l1fast[3];
+#pragma unroll
+        for (int j = 0; j < 3; ++j) l1fast[j] = l1base[j] - (kL1RowsHalf - 1) * h * kL1RowPitch * G::EB;
+        conv1_fast_pass<P>(smem, fast1_weights(b), r1, l1fast, a0);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 3; ++j) a0[0][j] = b0[0];
+        preload_ring<L1Pipe<P>::D, 1>(r1, layer_weights<P, 0>(packed, lane));
+        conv1_pass<P>(smem, layer_weights<P, 0>(packed, lane), r1, l1base, a0);
+      }
     }
-    conv1_pass<P>(smem, layer_weights<P, 0>(packed, lane), r1, l1base, a0);
     preload_flat<kRing>(r2, layer_weights<P, 1>(packed, lane));
     C6_MARK(2);
     pipe_layer<P, 1>(smem, packed, tail_lds, r2, ci, h, lane, wave, trace_on, lo_scale_w, a0, a1, [&] {
@@ -1351,11 +1432,7 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
       asm volatile("" : "+v"(hb));  // (one address register for all head weights)
       const float *pwg = reinterpret_cast<const float *>(smem + hb);
       const float *tl = pwg - 4 * h - kBiasTotal;
-      // The next board's input is asked for here: the counter of loads in flight is served in
-      // order, so in front of a K-loop these loads from HBM would hold up its weight fragments,
-      // while the heads wait for no load at all.
-      if (bn < b_end) issue_fetch(bn);
-      if (bn < b_end) preload_ring<L1Pipe<P>::D, 1>(r1, layer_weights<P, 0>(packed_of(bn), lane));
+      if (bn < b_end) preload_ring<L1Pipe<P>::D, 1>(r1, fast1_weights(bn));
       float pol[3] = {0.0f, 0.0f, 0.0f};
       float vsum = 0.0f;
 #pragma unroll
@@ -1391,6 +1468,11 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
       vsum = wave_sum(vsum);
       if (lane == 0) red[wave] = vsum;
       __syncthreads();
+      // The next board's input is asked for here, behind the board's last barrier but one (a
+      // barrier waits for loads that write LDS) and with no K-loop ahead: the counter of loads in
+      // flight is served in order, so in front of a K-loop these loads from HBM would hold up
+      // its weight fragments.
+      if (bn < b_end) issue_fetch(bn);
       if (tid == 0 && prm.value != nullptr) {
         float s = 0.0f;
 #pragma unroll
@@ -1711,8 +1793,42 @@ template <class P> __global__ void pack_kernel(const PackParams prm) {
     unsigned char *dst = prm.packed + (size_t)gid * 16;
     int l = 0;
     while (l < 8 && frag >= G::frag_offset(l + 1)) ++l;  // frag_offset is monotone
-    if (l >= 8) {  // over-read padding, or the fp8 weight copy behind it
+    if (l >= 8) {  // over-read padding, the low-order weight copies behind it, the second first-layer copy
       v4i o = {0, 0, 0, 0};
+      if (G::FAST1_FRAGS > 0 && frag >= G::PLANE2_FRAG_OFF && frag < G::PLANE2_FRAG_OFF + G::PLANE2_FRAGS) {
+        // the third plane's weights that fall inside the board, summed, as seen from the lane's
+        // output square: four channels per lane and fragment
+        const int fi = frag - G::PLANE2_FRAG_OFF, wv = fi / 12, j = (fi / 4) % 3, q = fi % 4;
+        int p = wv * kPixPerWave + j * 32 + m;
+        p = p < kPix ? p : kPix - 1;
+        const int r = p / kBoard, c = p % kBoard;
+        f32x4 t4;
+        for (int e = 0; e < 4; ++e) {
+          const float *w = prm.conv_w[0] + (size_t)((8 * q + 4 * h + e) * 3 + 2) * kK1 * kK1;
+          float sum = 0.0f;
+          for (int ky = 0; ky < kK1; ++ky) {
+            const int rr = r + ky - kK1 / 2;
+            if (rr < 0 || rr >= kBoard) continue;
+            for (int kx = 0; kx < kK1; ++kx) {
+              const int cc = c + kx - kK1 / 2;
+              if (cc >= 0 && cc < kBoard) sum += w[ky * kK1 + kx];
+            }
+          }
+          t4[e] = sum * act_scale<P>();
+        }
+        *reinterpret_cast<f32x4 *>(dst) = t4;
+        return;
+      }
+      if (G::FAST1_FRAGS > 0 && frag >= G::FAST1_OFF && frag < G::FAST1_OFF + G::FAST1_STEPS) {
+        // k-step (ky, 8 columns); lane half = input plane
+        const int fi = frag - G::FAST1_OFF, ky = fi / G::CPR, jj = fi % G::CPR;
+        const float *w = prm.conv_w[0];
+        for (int e = 0; e < G::E; ++e) {
+          const int kx = jj * G::E + e;
+          put_elem<P>(dst, e, kx < kK1 ? w[((m * 3 + h) * kK1 + ky) * kK1 + kx] * act_scale<P>() : 0.0f);
+        }
+        return;
+      }
       if constexpr (P::LO8) {
         int ll = 1;
         while (ll < 8 && frag >= G::lo_frag_offset(ll + 1)) ++ll;

@@ -134,7 +134,8 @@ def _bf16_round(t: torch.Tensor) -> torch.Tensor:
 
 
 def forward_bf16_emulated(
-    state: Mapping[str, torch.Tensor], x: torch.Tensor, act_scale: float = 1.0
+    state: Mapping[str, torch.Tensor], x: torch.Tensor, act_scale: float = 1.0,
+    exact_constant_plane: bool = False,
 ) -> tuple[torch.Tensor, torch.Tensor]:
     """The arithmetic contract of the bf16 HIP paths, emulated in fp32 torch:
     conv weights and layer inputs rounded to bf16 (RNE), fp32 accumulation,
@@ -144,13 +145,29 @@ def forward_bf16_emulated(
     ``act_scale`` c != 1 models the fused kernel, which carries c * activation
     between layers (c = -log2 e): first-layer weights are rounded AFTER the
     scaling, later layers see bf16(c * silu), biases are c * b in fp32, and the
-    heads divide the factor out again.  Mathematically the same network."""
+    heads divide the factor out again.  Mathematically the same network.
+
+    ``exact_constant_plane`` models the pipelined kernel's first layer: on a board whose last
+    input plane is one constant, that plane's weights are summed per output square in fp32
+    (unrounded) instead of going through the bf16 contraction."""
     n = _num_layers(state)
     c = float(act_scale)
     f = _bf16_round(x)
     for i in range(n):
         w = state[f"convs.{i}.weight"]
         wq = _bf16_round(w * c) if i == 0 else _bf16_round(w)
+        if i == 0 and exact_constant_plane:
+            last = x[:, -1]
+            const = (last == last[:, :1, :1]).flatten(1).all(dim=1).view(-1, 1, 1, 1)
+            wmix = wq.clone()
+            wmix[:, -1] = w[:, -1] * c      # the constant plane's weights unrounded ...
+            u_exact = F.conv2d(torch.cat((f[:, :-1], x[:, -1:]), 1), wmix, state["convs.0.bias"] * c,
+                               stride=1, padding=w.shape[-1] // 2)   # ... times its unrounded value
+            u_plain = F.conv2d(f, wq, state["convs.0.bias"] * c, stride=1, padding=w.shape[-1] // 2)
+            u = torch.where(const, u_exact, u_plain)
+            f = c * F.silu(u / c)
+            f = _bf16_round(f)
+            continue
         u = F.conv2d(f, wq, state[f"convs.{i}.bias"] * c, stride=1, padding=w.shape[-1] // 2)
         f = c * F.silu(u / c)
         if i + 1 < n:

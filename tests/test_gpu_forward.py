@@ -110,7 +110,7 @@ def test_16bit_paths_match_fp32_oracle_b4096(cuda, oracle_cfg2, init, prec):
         # arithmetic emulated in fp32 PyTorch (oracle.forward_bf16_emulated) gives 97-99 %.
         # The kernel must do no worse than that emulation, and match it closely.
         with torch.inference_mode():
-            le, _ = R.forward_bf16_emulated(st, x, act_scale=-1.4426950408889634)
+            le, _ = R.forward_bf16_emulated(st, x, act_scale=-1.4426950408889634, exact_constant_plane=True)
         emu = argmax_agreement(R.mask_logits(le, legal), R.mask_logits(lo, legal))
         assert agree >= emu - 0.005
         assert rel_l2(lg, le) <= 5e-3
@@ -420,3 +420,26 @@ def test_phase_profile_runs_when_the_traced_library_is_built(cuda):
                          text=True, timeout=280)
     assert out.returncode == 0, out.stderr[-2000:]
     assert "one board =" in out.stdout and "conv8 low-order pass" in out.stdout
+
+
+@pytest.mark.parametrize("prec", ["bf16f6", "bf16", "fp16"])
+def test_first_layer_paths_constant_and_varying_third_plane(cuda, prec):
+    """The pipelined kernel runs the first layer on two planes plus a per-square table when a
+    board's third plane is one constant (what the reference feeds it) and on all three planes
+    otherwise; the choice is made per board.  Both against the fp32 oracle, mixed in one batch."""
+    st = R.init_state(21, "reference")
+    x, legal = gen_boards(96, 200, 17)
+    g = torch.Generator().manual_seed(5)
+    x = x.clone()
+    x[0::3, 2] = torch.rand(32, 19, 19, generator=g)            # varying plane
+    x[1::3, 2] = 0.37                                          # constant, neither 0 nor 1
+    x[2::3, :2] += 0.25 * torch.rand(32, 2, 19, 19, generator=g)  # non-binary stones, constant third plane
+    with torch.inference_mode():
+        lo, vo = R.forward(st, x)
+        lg, vg = make_model(cuda, st, prec)(x.to(cuda))
+    for sel in (slice(0, None, 3), slice(1, None, 3), slice(2, None, 3)):
+        assert rel_l2(lg[sel], lo[sel]) <= BF16_TOL and rel_l2(vg[sel], vo[sel]) <= BF16_TOL
+    # a board evaluates the same alone and inside the mixed batch
+    with torch.inference_mode():
+        one, _ = make_model(cuda, st, prec)(x[:1].to(cuda))
+    assert torch.equal(one[0], lg[0])

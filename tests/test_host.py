@@ -63,8 +63,11 @@ def test_packed_sizes_follow_the_layout():
             n += (9 * cin // kstep) * (cout // 32)
         return n + 24
     tail = (544 + 96 + 96 + 4 + 8) * 4
-    assert _lib.packed_bytes(_lib.PREC_BF16) == frags(8) * 1024 + tail
-    assert _lib.packed_bytes(_lib.PREC_F16) == frags(8) * 1024 + tail
+    # pipelined modes: plus the first layer's two-plane copy (23 rows x 3 fragments, 8 over-read)
+    # and the third plane's table as the lanes hold it (4 waves x 3 pixel tiles x 4 quads)
+    fast1 = 23 * 3 + 8 + 4 * 3 * 4
+    assert _lib.packed_bytes(_lib.PREC_BF16) == (frags(8) + fast1) * 1024 + tail
+    assert _lib.packed_bytes(_lib.PREC_F16) == (frags(8) + fast1) * 1024 + tail
     assert _lib.packed_bytes(_lib.PREC_BF16X2) == frags(8) * 1024 + tail
     assert _lib.packed_bytes(_lib.PREC_F32) == frags(4) * 1024 + tail
     # bf16 + fp8: plus the e4m3 copy of the 3x3 layers (64-wide chunks, two 16-byte pieces per lane)
@@ -72,7 +75,7 @@ def test_packed_sizes_follow_the_layout():
     for cin, cout in zip((32, 32, 64, 64, 64, 96, 96), (32, 64, 64, 64, 96, 96, 96)):
         lo += ((9 * cin // 32 + 1) // 2) * (cout // 32) * 2
     assert _lib.packed_bytes(_lib.PREC_BF16F8) == (frags(8) + lo + 18) * 1024 + tail
-    assert _lib.packed_bytes(_lib.PREC_BF16F6) == _lib.packed_bytes(_lib.PREC_BF16F8)  # same fragment grid
+    assert _lib.packed_bytes(_lib.PREC_BF16F6) == _lib.packed_bytes(_lib.PREC_BF16F8) + fast1 * 1024
     with pytest.raises(ValueError):
         _lib.packed_bytes(9)
 
