@@ -1276,6 +1276,7 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
   // third plane; a board that has none refills it)
   preload_ring<L1Pipe<P>::D, 1>(r1, fast1_weights(b));
   issue_fetch(b);
+  if (tid == 0) reinterpret_cast<int *>(red)[8] = 0;  // (the first board's flag, see the staging)
 
   for (; b < b_end; ++b) {
     int tidv = tid;  // opaque per board: keeps per-thread staging addresses out of long-lived registers
@@ -1330,15 +1331,25 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
       __builtin_amdgcn_sched_barrier(0);  // (issue here)
     }
     // ---- stage the input: zero the shifted copies, then scatter the board ----
-    int *plane2_flag = reinterpret_cast<int *>(red) + 8;  // set by any thread that sees the third plane vary
-    if (tid == 0) *plane2_flag = 0;
+    // Does the third plane vary?  Any thread that sees it differ from square 0 raises this board's
+    // flag (two flags, used in turn: the other one is cleared for the next board meanwhile).
+    int *plane2_flag = reinterpret_cast<int *>(red) + 8 + (int)((b - b_first) & 1);
+    {
+      bool varies = false;
+#pragma unroll
+      for (int r = 0; r < ROUNDS; ++r)
+        if (tidv + r * THREADS < kPix) varies |= plane2_differs(tidv + r * THREADS);
+      if (varies) *plane2_flag = 1;
+      if (tid == 0) reinterpret_cast<int *>(red)[8 + (int)((b - b_first + 1) & 1)] = 0;
+    }
     {
       const v4i z = {0, 0, 0, 0};
       for (int i = tidv * 16; i < G::COPIES_BYTES; i += THREADS * 16)
         *reinterpret_cast<v4i *>(smem + i) = z;
     }
     __syncthreads();
-    bool varies = false;
+    const bool plane2_varies = *plane2_flag != 0;
+    const int planes_staged = plane2_varies ? 3 : 2;  // (a constant third plane is not contracted)
 #pragma unroll
     for (int r = 0; r < ROUNDS; ++r) {
       const int p = tidv + r * THREADS;
@@ -1347,10 +1358,10 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
         float v[3];
         unsigned o;
         staged_input(p, v, o);
-        varies |= plane2_differs(p);
         occ[p] = (unsigned char)o;
 #pragma unroll
         for (int ch = 0; ch < 3; ++ch) {
+          if (ch >= planes_staged) break;
           const int hrow = (row + kK1 / 2) * 3 + ch;
           const unsigned short v16 = bits16<P>(v[ch]);
 #pragma unroll
@@ -1367,9 +1378,7 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
         if (tidv + r * THREADS < TAILN)
           reinterpret_cast<float *>(smem + G::TAIL_LDS_OFF)[tidv + r * THREADS] = tailv[r];
     }
-    if (varies) *plane2_flag = 1;
     __syncthreads();
-    const bool plane2_varies = *plane2_flag != 0;
     C6_MARK(1);
 
     v4i r2[kRing], r3[kRing * 2], r6[kRing * 3];  // weight rings of layers 2, 3-5, 6-8
