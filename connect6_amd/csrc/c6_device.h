@@ -6,6 +6,13 @@
 
 namespace c6 {
 
+// A non-temporal store, for an output that is streamed to HBM and not read again here.  Measured
+// on 0.85 GB of masked logits it is worth 3 %; the view gather gains nothing from it and the
+// canonical planes lose 7 %, so only the masking kernels use it.
+template <class T> __device__ __forceinline__ void stream_store(T *p, const T &v) {
+  __builtin_nontemporal_store(v, p);
+}
+
 // Wave64 all-reduce without LDS traffic: DPP inside a row of 16 lanes (quad swaps, then the
 // mirrored lane of the 8- and the 16-group, which belongs to the half not yet combined), then
 // v_permlane16_swap / v_permlane32_swap across rows.  Every lane ends with the result.

@@ -918,19 +918,20 @@ __device__ __forceinline__ void epi_atom(unsigned char *smem, const int (&wb)[3]
       // slot 2i <- first[i], slot 2i+1 <- second[i]; only slots 0-15 (i < 8) are kept.  The upper
       // halves are never used, but the instruction reads them: left undefined they get registers
       // that weight loads in flight are about to write, and the hardware then waits for every
-      // such load before the conversion.  So `first` is the lane's 16 values in order (its upper
-      // half is what `second` starts with), and the upper half of `second` is eight registers
-      // that an empty asm statement "defines".
+      // such load before the conversion.  So the upper half of each operand is eight registers
+      // that an empty asm statement "defines" (no instruction; they are only reserved for the
+      // length of the conversion).
       typedef float f32x8v __attribute__((ext_vector_type(8)));
-      f32x8v p0, p1, fill;
+      f32x8v p0, p1, fill0, fill1;
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         p0[i] = c.lo[b][i];
         p1[i] = c.lo[b][8 + i];
       }
-      asm volatile("" : "=v"(fill));
-      const f32x16v first = __builtin_shufflevector(p0, p1, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
-      const f32x16v second = __builtin_shufflevector(p1, fill, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
+      asm volatile("" : "=v"(fill0));
+      asm volatile("" : "=v"(fill1));
+      const f32x16v first = __builtin_shufflevector(p0, fill0, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
+      const f32x16v second = __builtin_shufflevector(p1, fill1, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
       const u32x6 r = to_fp6_block(first, second, __builtin_bit_cast(float, c.sc[b] << 23));
       unsigned char *dst = smem + wb[j] + G::LO_OFF + 32 * t;  // + 8h from wb: data at + 4h more = 12h
       // (three dwords at a 4-byte aligned address: dword stores)

@@ -20,7 +20,7 @@ __global__ void mask4_kernel(const uint32_t *__restrict__ in, const uint8_t *__r
     o[1] = (m & 0x0000ff00u) ? v[1] : (int)fill;
     o[2] = (m & 0x00ff0000u) ? v[2] : (int)fill;
     o[3] = (m & 0xff000000u) ? v[3] : (int)fill;
-    reinterpret_cast<v4i *>(out)[i] = o;
+    stream_store(&reinterpret_cast<v4i *>(out)[i], o);
   }
   if (blockIdx.x == 0 && threadIdx.x < (n & 3)) {
     const long long i = (nv << 2) + threadIdx.x;
@@ -44,7 +44,7 @@ __global__ void mask2_kernel(const uint16_t *__restrict__ in, const uint8_t *__r
       const uint32_t hi = (mm & 0xff00u) ? ((uint32_t)v[w] >> 16) : (uint32_t)fill;
       o[w] = (int)(lo | (hi << 16));
     }
-    reinterpret_cast<v4i *>(out)[i] = o;
+    stream_store(&reinterpret_cast<v4i *>(out)[i], o);
   }
   if (blockIdx.x == 0 && threadIdx.x < (n & 7)) {
     const long long i = (nv << 3) + threadIdx.x;
