@@ -682,9 +682,11 @@ template <int N>
 __device__ __forceinline__ void load_bias_tiles_lds(f32x16 (&bt)[N], const unsigned char *smem,
                                                     int tail_lds, int layer_off, int h) {
   // one address register, made opaque here: otherwise every address below is computed once per
-  // kernel, kept in a register of its own and ends up in scratch memory
-  int base = tail_lds + 4 * layer_off + 16 * h;
+  // kernel, kept in a register of its own and ends up in scratch memory (and so would the sum
+  // below, per layer, were the layer's constant added in front of the asm statement)
+  int base = 16 * h;
   asm volatile("" : "+v"(base));
+  base += tail_lds + 4 * layer_off;
 #pragma unroll
   for (int t = 0; t < N; ++t)
 #pragma unroll
@@ -1158,20 +1160,24 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
   const int h = lane >> 5;
   const int n = lane & 31;
 
-  // per-lane pixel geometry of the three 32-pixel tiles of this quarter
-  int ci[3], l1base[3], pix[3];
-  bool valid[3];
+  // Per-lane pixel geometry of the three 32-pixel tiles of this quarter.  Only the activation
+  // tile's position index lives through the kernel; what the first layer and the heads need is
+  // recomputed per board from an opaque copy of the thread index (a dozen instructions), since
+  // values kept from here to there end up in scratch memory.
+  auto tile_pixel = [](int t, int j, bool &ok) __attribute__((always_inline)) {
+    const int p = (t >> 6) * kPixPerWave + j * 32 + (t & 31);
+    ok = p < kPix;
+    return ok ? p : (kPix - 1);
+  };
+  int ci[3];
 #pragma unroll
   for (int j = 0; j < 3; ++j) {
-    const int p = wave * kPixPerWave + j * 32 + n;
-    valid[j] = p < kPix;
-    const int pc = valid[j] ? p : (kPix - 1);
-    pix[j] = pc;
+    bool ok;
+    const int pc = tile_pixel(tid, j, ok);
     const int r = pc / kBoard, c = pc - r * kBoard;
     ci[j] = (r + 1) * kPitch + (c + 1);
-    const int s = c % G::E;
-    l1base[j] = s * G::COPY_BYTES + ((r * 3 + kL1RowsHalf * h) * kL1RowPitch + (c - s)) * G::EB;
   }
+  (void)n;
 
   unsigned char *occ = smem + G::OCC_OFF;
   float *lgt = reinterpret_cast<float *>(smem + G::LGT_OFF);
@@ -1191,41 +1197,45 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
     return src < 0 ? 0 : (src >= prm.num_states ? prm.num_states - 1 : src);
   };
   auto issue_fetch = [&](long long b) {
+    // (lane and wave opaque per call: the chunk addresses are then computed here and not kept,
+    // one register pair per chunk, for the whole kernel)
+    int ln = lane, wv = wave;
+    asm volatile("" : "+v"(ln), "+v"(wv));
     unsigned char *dst = smem + G::NEXT_IN_OFF;
     if (prm.x_dtype == C6_DT_BOARD_I8) {
       // environment state (connect6/vector_env.py:196-218 of the reference), seen through D4
       // view prm.view (connect6/train.py:222-230): the stones, the side to move, stones left
       const long long src = board_row(b);
       const int8_t *board = reinterpret_cast<const int8_t *>(prm.x) + (size_t)src * kPix;
-      for (int i = wave; i < (kPix + 63) / 64; i += NWAVES) {
-        const int p = i * 64 + lane;
+      for (int i = wv; i < (kPix + 63) / 64; i += NWAVES) {
+        const int p = i * 64 + ln;
         if (p < kPix)
           __builtin_amdgcn_global_load_lds((GPtr)(board + (prm.view ? d4_from_view(p, prm.view) : p)),
                                            (LPtr)(dst + (G::NEXT_IN_BYTES_AT + i * 64) * 4), 1, 0, 0);
       }
-      if (wave == 0 && lane < 2)
-        __builtin_amdgcn_global_load_lds((GPtr)((lane == 0 ? prm.player : prm.stones_left) + src),
+      if (wv == 0 && ln < 2)
+        __builtin_amdgcn_global_load_lds((GPtr)((ln == 0 ? prm.player : prm.stones_left) + src),
                                          (LPtr)(dst + G::NEXT_IN_AUX * 4), 1, 0, 0);
       return;
     }
     constexpr int NE = 3 * kPix;
     if (prm.x_dtype == C6_DT_F32) {
       const float *xf = reinterpret_cast<const float *>(prm.x) + (size_t)b * NE;
-      for (int i = wave; i < (NE + 63) / 64; i += NWAVES) {
-        const int e = i * 64 + lane;
+      for (int i = wv; i < (NE + 63) / 64; i += NWAVES) {
+        const int e = i * 64 + ln;
         if (e < NE) __builtin_amdgcn_global_load_lds((GPtr)(xf + e), (LPtr)(dst + i * 256), 4, 0, 0);
       }
     } else {
       const unsigned short *xh = reinterpret_cast<const unsigned short *>(prm.x) + (size_t)b * NE;
-      for (int i = wave; i < (NE + 63) / 64; i += NWAVES) {
-        const int e = i * 64 + lane;
+      for (int i = wv; i < (NE + 63) / 64; i += NWAVES) {
+        const int e = i * 64 + ln;
         if (e < NE) __builtin_amdgcn_global_load_lds((GPtr)(xh + e), (LPtr)(dst + i * 256), 2, 0, 0);
       }
     }
     if (prm.mask_mode == C6_MASK_LEGAL) {
       const uint8_t *lg = prm.legal + (size_t)b * kPix;
-      for (int i = wave; i < (kPix + 63) / 64; i += NWAVES) {
-        const int p = i * 64 + lane;
+      for (int i = wv; i < (kPix + 63) / 64; i += NWAVES) {
+        const int p = i * 64 + ln;
         if (p < kPix)
           __builtin_amdgcn_global_load_lds((GPtr)(lg + p), (LPtr)(dst + (G::NEXT_IN_BYTES_AT + i * 64) * 4), 1, 0, 0);
       }
@@ -1284,15 +1294,9 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
     asm volatile("" : "+v"(tidv));
     const unsigned char *packed = packed_of(b);
     const float *tail = reinterpret_cast<const float *>(packed + G::TAIL_OFF);
-    // the weight set's fp32 tail goes to LDS whenever the set changes
-    constexpr int TAILN = kBiasTotal + 2 * kHeadC + 4, TAILR = (TAILN + THREADS - 1) / THREADS;
+    // the weight set's fp32 tail goes to LDS whenever the set changes (see the staging)
+    constexpr int TAILN = kBiasTotal + 2 * kHeadC + 4;
     const bool new_set = b == b_first || packed != packed_of(b - 1);
-    float tailv[TAILR];
-    if (new_set) {
-#pragma unroll
-      for (int r = 0; r < TAILR; ++r)
-        if (tidv + r * THREADS < TAILN) tailv[r] = tail[tidv + r * THREADS];
-    }
     const int tail_lds = G::TAIL_LDS_OFF;
     // block-scale exponents of the low-order weight copies (E8M0: 127 - log2 of the copy's scale),
     // fetched here, long before any second pass needs them
@@ -1374,10 +1378,14 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
       }
     }
     if (new_set) {
-#pragma unroll
-      for (int r = 0; r < TAILR; ++r)
-        if (tidv + r * THREADS < TAILN)
-          reinterpret_cast<float *>(smem + G::TAIL_LDS_OFF)[tidv + r * THREADS] = tailv[r];
+      // straight into LDS, 64 floats per instruction (lane l's float lands in word l behind the
+      // instruction's base); the barrier below waits for loads that write LDS
+      for (int i = tidv >> 6; i < (TAILN + 63) / 64; i += NWAVES) {
+        const int e = i * 64 + (tidv & 63);
+        if (e < TAILN)
+          __builtin_amdgcn_global_load_lds((GPtr)(tail + e), (LPtr)(smem + G::TAIL_LDS_OFF + i * 256), 4, 0, 0);
+      }
+      __builtin_amdgcn_s_waitcnt(0);  // landed before this wave reaches the barrier
     }
     __syncthreads();
     C6_MARK(1);
@@ -1386,6 +1394,14 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
     f32x16 a1[1][3];
     // ---- layer 1 ----
     {
+      int l1base[3];
+#pragma unroll
+      for (int j = 0; j < 3; ++j) {
+        bool ok;
+        const int pc = tile_pixel(tidv, j, ok);
+        const int r = pc / kBoard, c = pc - r * kBoard, s = c % G::E;
+        l1base[j] = s * G::COPY_BYTES + ((r * 3 + kL1RowsHalf * ((tidv >> 5) & 1)) * kL1RowPitch + (c - s)) * G::EB;
+      }
       f32x16 b0[1];
       load_bias_tiles_lds(b0, smem, tail_lds, bias_offset(0), h);
       if (!plane2_varies) {
@@ -1442,6 +1458,10 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
       asm volatile("" : "+v"(hb));  // (one address register for all head weights)
       const float *pwg = reinterpret_cast<const float *>(smem + hb);
       const float *tl = pwg - 4 * h - kBiasTotal;
+      int pix[3];
+      bool valid[3];
+#pragma unroll
+      for (int j = 0; j < 3; ++j) pix[j] = tile_pixel(tidv, j, valid[j]);
       if (bn < b_end) preload_ring<L1Pipe<P>::D, 1>(r1, fast1_weights(bn));
       float pol[3] = {0.0f, 0.0f, 0.0f};
       float vsum = 0.0f;
@@ -1494,17 +1514,20 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
 
     // ---- write out: masked logits, optional sampled action ----
     if (prm.logits != nullptr) {
-      for (int p = tid; p < kPix; p += THREADS) {
+      for (int p = tidv; p < kPix; p += THREADS) {
         const float v = lgt[p];
         prm.logits[(size_t)b * kPix + p] = occ[p] ? prm.fill : v;
       }
     }
     if (prm.actions != nullptr && wave == 0) {
-      const float it = prm.inv_temperature;
+      float it = prm.inv_temperature;
+      asm volatile("" : "+s"(it));  // (what is derived from it is derived here, not kept)
       int a;
       float lp;
+      int lane_here = lane;  // opaque per board: the entries' LDS addresses are computed here,
+      asm volatile("" : "+v"(lane_here));  // not once per kernel into registers that get spilled
       wave_sample(
-          lane, prm.u[b], it, [&](int i) { return lgt[i]; }, [&](int i) { return occ[i] == 0; },
+          lane_here, prm.u[b], it, [&](int i) { return lgt[i]; }, [&](int i) { return occ[i] == 0; },
           a, lp);
       if (lane == 0) {
         prm.actions[b] = a;
