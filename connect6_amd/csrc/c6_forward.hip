@@ -495,7 +495,9 @@ __device__ __forceinline__ void lo_preload(v4i (&f0)[D][NT], v4i (&f1)[D][NT],
 // A runtime loop over groups of D chunks (D = ring depth) keeps the compiler from hoisting
 // every fragment load of the layer to the front.
 //   INIT: the accumulators are undefined on entry; the first chunk's MFMAs start from `bias`
-template <class P, int L, bool INIT, int D, int NT>
+//   BYTE_BASE: `ci` holds byte addresses (position record + 8 * lane half, what the epilogue
+//   stores through) instead of position indices: no address registers of the pass's own
+template <class P, int L, bool INIT, bool BYTE_BASE, int D, int NT>
 __device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
                                               const unsigned char *packed, int scale_w,
                                               v4i (&ring0)[D][NT], v4i (&ring1)[D][NT],
@@ -515,17 +517,20 @@ __device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
 
   int pbase[3];
 #pragma unroll
-  for (int j = 0; j < 3; ++j) pbase[j] = ci[j] * G::PIXB + G::LO_OFF;
-  // byte offset of this lane half's half-chunk of chunk c, relative to the centre position
+  for (int j = 0; j < 3; ++j) pbase[j] = BYTE_BASE ? ci[j] : ci[j] * G::PIXB + G::LO_OFF;
+  // byte offset of this lane half's half-chunk of chunk c, relative to pbase[]
   auto half_off = [&](int c) {
     int g = 2 * c + h;
     g = g < HC ? g : HC - 1;  // the padding half-chunk re-reads the last one (its weights are zero)
     const int tap = g / PER32, cb = g - tap * PER32;
     const int ky = tap / 3, kx = tap - 3 * ky;
-    return ((ky - 1) * kPitch + (kx - 1)) * G::PIXB + cb * 32;
+    return ((ky - 1) * kPitch + (kx - 1)) * G::PIXB + cb * 32 + (BYTE_BASE ? G::LO_OFF - 8 * h : 0);
   };
   auto fetch = [&](int c, v4i (&b)[3][2]) {
-    const int off = half_off(c);
+    // (opaque: the sums with pbase[] are then formed here, three additions, and not once per
+    // kernel for every unrolled chunk, in registers that end up in scratch memory)
+    int off = half_off(c);
+    asm volatile("" : "+v"(off));
 #pragma unroll
     for (int j = 0; j < 3; ++j) {
       b[j][0] = *reinterpret_cast<const v4i *>(smem + pbase[j] + off);
@@ -725,7 +730,7 @@ __device__ __forceinline__ void mid_layer(
     lo_preload<P, L>(lor0, lor1, packed, lane);
     {
       f32x16 nobias[NT];
-      conv3_lo_pass<P, L, false>(smem, packed, lo_scale_w[L], lor0, lor1, ci, h, lane, acc, nobias);
+      conv3_lo_pass<P, L, false, false>(smem, packed, lo_scale_w[L], lor0, lor1, ci, h, lane, acc, nobias);
     }
   }
   // With equal channel counts the main pass's over-read has already left the next layer's first
@@ -1127,7 +1132,7 @@ __device__ __forceinline__ void pipe_layer(
   });
   C6_MARK(30 + L);
   if constexpr (kLoPass) {
-    conv3_lo_pass<P, L, NTP == 1>(smem, packed, lo_scale_w[L], lor0, lor1, ci, h, lane, acc, bias);
+    conv3_lo_pass<P, L, NTP == 1, true>(smem, packed, lo_scale_w[L], lor0, lor1, wb, h, lane, acc, bias);
     // before part B overwrites fp6 block 0, every wave must have read it
     if constexpr (NT > 1 && !kLast) __syncthreads();
   }
@@ -1727,7 +1732,7 @@ __global__ __launch_bounds__(256) void fused_forward_kernel(const FwdParams prm)
       if constexpr (P::LO8) lo_preload<P, 7>(lor0, lor1, packed, lane);
       if constexpr (P::LO8) {
         f32x16 nobias[3];
-        conv3_lo_pass<P, 7, false>(smem, packed, lo_scale_w[7], lor0, lor1, ci, h, lane, acc, nobias);
+        conv3_lo_pass<P, 7, false, false>(smem, packed, lo_scale_w[7], lor0, lor1, ci, h, lane, acc, nobias);
       }
       if (bn < b_end) preload_ring<L1Pipe<P>::D, 1>(r1, layer_weights<P, 0>(packed_of(bn), lane));
       C6_MARK(18);
