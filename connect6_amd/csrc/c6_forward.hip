@@ -1353,9 +1353,16 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
       if (tid == 0) reinterpret_cast<int *>(red)[8 + (int)((b - b_first + 1) & 1)] = 0;
     }
     {
+      // (unrolled, one address register and immediate offsets: as a loop the same stores take
+      // twice as long, 2.0 k cycles against 1.1 k measured alone -- LDS stores are bound by the
+      // wave's own instruction issue here)
       const v4i z = {0, 0, 0, 0};
-      for (int i = tidv * 16; i < G::COPIES_BYTES; i += THREADS * 16)
-        *reinterpret_cast<v4i *>(smem + i) = z;
+      constexpr int WHOLE = G::COPIES_BYTES / 16 / THREADS;
+      unsigned char *zp = smem + tidv * 16;
+#pragma unroll
+      for (int u = 0; u < WHOLE; ++u) *reinterpret_cast<v4i *>(zp + u * (THREADS * 16)) = z;
+      if (tidv * 16 + WHOLE * (THREADS * 16) < G::COPIES_BYTES)
+        *reinterpret_cast<v4i *>(zp + WHOLE * (THREADS * 16)) = z;
     }
     __syncthreads();
     const bool plane2_varies = *plane2_flag != 0;
