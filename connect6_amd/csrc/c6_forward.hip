@@ -518,19 +518,64 @@ __device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
   int pbase[3];
 #pragma unroll
   for (int j = 0; j < 3; ++j) pbase[j] = BYTE_BASE ? ci[j] : ci[j] * G::PIXB + G::LO_OFF;
-  // byte offset of this lane half's half-chunk of chunk c, relative to pbase[]
-  auto half_off = [&](int c) {
-    int g = 2 * c + h;
-    g = g < HC ? g : HC - 1;  // the padding half-chunk re-reads the last one (its weights are zero)
-    const int tap = g / PER32, cb = g - tap * PER32;
-    const int ky = tap / 3, kx = tap - 3 * ky;
-    return ((ky - 1) * kPitch + (kx - 1)) * G::PIXB + cb * 32 + (BYTE_BASE ? G::LO_OFF - 8 * h : 0);
+  // Byte offset of a half-chunk relative to pbase[].  Half-chunk g = 2 c + (lane half) of chunk
+  // c = 3 grp + dd is g = 6 grp + r with r = 2 dd + half: with `r` a constant, the tap and the
+  // channel block of g need no division by the tile count, and for 64 input channels (6
+  // half-chunks = 3 taps = one kernel row) no division at all.  The group number may be a
+  // run-time value (scalar unit); both halves' offsets are formed and the lane half selects.
+  // (The lane half through an opaque copy: the selected offsets of the unrolled chunks are then
+  // formed in this pass and not once per kernel, in registers that get spilled.)
+  static_assert(D == 3, "the half-chunk arithmetic below assumes groups of three chunks");
+  int hh = h;
+  asm volatile("" : "+v"(hh));
+  auto off_g = [&](int grp, int r) __attribute__((always_inline)) {
+    int ky, kx, cb;
+    if constexpr (PER32 == 3) {
+      const unsigned tap = 2u * (unsigned)grp + (unsigned)(r / 3);
+      cb = r % 3;
+      ky = (int)(tap / 3u);
+      kx = (int)tap - 3 * ky;
+    } else if constexpr (PER32 == 2) {
+      cb = r % 2;
+      ky = grp + (r / 2) / 3;
+      kx = (r / 2) % 3;
+    } else {
+      static_assert(PER32 == 1, "32, 64 or 96 input channels");
+      cb = 0;
+      ky = 2 * grp + r / 3;
+      kx = r % 3;
+    }
+    return ((ky - 1) * kPitch + (kx - 1)) * G::PIXB + cb * 32 + (BYTE_BASE ? G::LO_OFF : 0);
   };
-  auto fetch = [&](int c, v4i (&b)[3][2]) {
-    // (opaque: the sums with pbase[] are then formed here, three additions, and not once per
-    // kernel for every unrolled chunk, in registers that end up in scratch memory)
-    int off = half_off(c);
-    asm volatile("" : "+v"(off));
+  // chunk 3 grp + dd; STATIC: grp is a constant after unrolling, and the chunk may lie beyond the
+  // last one (harmless re-reads of the last) or hold the padding half-chunk (which re-reads the
+  // half-chunk before it: its weights are zero)
+  auto fetch = [&](int grp, int dd, auto is_static, v4i (&b)[3][2]) __attribute__((always_inline)) {
+    auto of_chunk = [&](int c, int &o0, int &o1) __attribute__((always_inline)) {  // constant c
+      c = c < NC ? c : NC - 1;
+      const int g0 = 2 * c, g1 = 2 * c + 1 < HC ? 2 * c + 1 : HC - 1;
+      o0 = off_g(g0 / 6, g0 % 6);
+      o1 = off_g(g1 / 6, g1 % 6);
+    };
+    int o0, o1;
+    if constexpr (!BYTE_BASE) {
+      // (the layer-by-layer kernels: one formula on the lane's own half-chunk number; the
+      // scalar form below costs them registers)
+      int c = D * grp + dd;
+      c = c < NC ? c : NC - 1;
+      int g = 2 * c + hh;
+      g = g < HC ? g : HC - 1;
+      const int tap = g / PER32, cb = g - tap * PER32;
+      const int ky = tap / 3, kx = tap - 3 * ky;
+      o0 = o1 = ((ky - 1) * kPitch + (kx - 1)) * G::PIXB + cb * 32;
+    } else if constexpr (decltype(is_static)::value) {
+      of_chunk(D * grp + dd, o0, o1);
+    } else {
+      // (run-time group: never the last chunk nor beyond it, see the loop bounds below)
+      o0 = off_g(grp, 2 * dd);
+      o1 = off_g(grp, 2 * dd + 1);
+    }
+    const int off = hh ? o1 - (BYTE_BASE ? 8 : 0) : o0;
 #pragma unroll
     for (int j = 0; j < 3; ++j) {
       b[j][0] = *reinterpret_cast<const v4i *>(smem + pbase[j] + off);
@@ -539,7 +584,7 @@ __device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
         // register that the compiler reuses at once, waiting for the read to land first)
         typedef int v3i __attribute__((ext_vector_type(3)));
         const v3i q = *reinterpret_cast<const v3i *>(smem + pbase[j] + off + 16);
-        b[j][1] = v4i{q[0], q[1], q[2], 0};
+        b[j][1] = v4i{q[0], q[1], q[2], q[2]};  // (register 7 is not read: no constant to move in)
       } else {
         b[j][1] = *reinterpret_cast<const v4i *>(smem + pbase[j] + off + 16);
       }
@@ -549,13 +594,13 @@ __device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
   static_assert(D % (kAhead + 1) == 0 && NC > kAhead, "low-order ring and fragment queue shapes");
   v4i bq[kAhead + 1][3][2];
 #pragma unroll
-  for (int a = 0; a < kAhead; ++a) fetch(a, bq[a]);
-  // chunk c0 + d: its MFMAs, the LDS reads of chunk c0 + d + kAhead and the refill of ring slot d
-  auto chunk = [&](int c0, int d, auto first) {
-    const WFrags wn = wl + (c0 + D) * NT * 2;
+  for (int a = 0; a < kAhead; ++a) fetch(0, a, IC<1>{}, bq[a]);
+  // chunk 3 grp + d: its MFMAs, the LDS reads of the chunk kAhead further on and the refill of
+  // ring slot d
+  auto chunk = [&](int grp, int d, auto first, auto is_static) __attribute__((always_inline)) {
+    const WFrags wn = wl + (grp + 1) * (D * NT * 2);
     v4i(&bcur)[3][2] = bq[d % (kAhead + 1)];
-    // (after the last chunks: harmless re-reads)
-    fetch(c0 + d + kAhead < NC ? c0 + d + kAhead : NC - 1, bq[(d + kAhead) % (kAhead + 1)]);
+    fetch(grp + (d + kAhead) / D, (d + kAhead) % D, is_static, bq[(d + kAhead) % (kAhead + 1)]);
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       const v8i a = __builtin_shufflevector(ring0[d][t], ring1[d][t], 0, 1, 2, 3, 4, 5, 6, 7);
@@ -583,21 +628,26 @@ __device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
   };
   // Whole groups of D chunks in a runtime loop with a single basic block (a branch inside the
   // body makes the compiler wait for every LDS read in flight at each group boundary), then the
-  // NC % D chunks that are left, unrolled.
-  constexpr int WHOLE = NC / D * D;
-  static_assert(WHOLE >= D, "at least one whole group");
+  // chunks that are left, unrolled.  With the scalar offsets (BYTE_BASE) the loop only takes the
+  // groups whose reads ahead stay in front of the last chunk, so that its body needs neither of
+  // the two special cases (a select per read costs more than the longer unrolled tail).
+  constexpr int LIM = NC - 2 - (D - 1) - kAhead;  // last chunk such a group may start at
+  constexpr int GROUPS = BYTE_BASE ? (LIM >= 0 ? LIM / D + 1 : 0) : NC / D;
+  constexpr int FIRST = INIT ? 1 : 0;
+  static_assert(NC >= D, "at least one whole group");
   if constexpr (INIT) {  // (the first group apart: its first chunk initialises the accumulators)
-    chunk(0, 0, IC<1>{});
+    chunk(0, 0, IC<1>{}, IC<1>{});
 #pragma unroll
-    for (int d = 1; d < D; ++d) chunk(0, d, IC<0>{});
+    for (int d = 1; d < D; ++d) chunk(0, d, IC<0>{}, IC<1>{});
   }
 #pragma unroll 1
-  for (int c0 = INIT ? D : 0; c0 < WHOLE; c0 += D) {
+  for (int grp = FIRST; grp < GROUPS; ++grp) {
 #pragma unroll
-    for (int d = 0; d < D; ++d) chunk(c0, d, IC<0>{});
+    for (int d = 0; d < D; ++d) chunk(grp, d, IC<0>{}, IC<0>{});
   }
+  constexpr int REST = (GROUPS > FIRST ? GROUPS : FIRST) * D;
 #pragma unroll
-  for (int d = 0; d < NC % D; ++d) chunk(WHOLE, d, IC<0>{});
+  for (int c = REST; c < NC; ++c) chunk(c / D, c % D, IC<0>{}, IC<1>{});
 }
 
 // SiLU of the four accumulators (tile t, pixel tile j, quad q): bias was added at init
@@ -1472,8 +1522,10 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
       const float *tl = pwg - 4 * h - kBiasTotal;
       int pix[3];
       bool valid[3];
+      int th = tidv;
+      asm volatile("" : "+v"(th));  // (computed here, not at the top of the board and kept)
 #pragma unroll
-      for (int j = 0; j < 3; ++j) pix[j] = tile_pixel(tidv, j, valid[j]);
+      for (int j = 0; j < 3; ++j) pix[j] = tile_pixel(th, j, valid[j]);
       if (bn < b_end) preload_ring<L1Pipe<P>::D, 1>(r1, fast1_weights(bn));
       float pol[3] = {0.0f, 0.0f, 0.0f};
       float vsum = 0.0f;
