@@ -87,6 +87,29 @@ def test_ragged_batches(cuda, batch):
     assert rel_l2(lg, lo) <= FP32_TOL and rel_l2(vg, vo) <= FP32_TOL
 
 
+@pytest.mark.parametrize("prec", ["bf16f6", "bf16", "fp16", "bf16f8"])
+def test_16bit_modes_on_ragged_batches(cuda, prec):
+    """A board's result does not depend on the batch around it: every prefix of a batch gives,
+    bit for bit, the rows of the whole batch (workgroups with one board, with none, with a
+    last board that has no successor to prefetch), masked logits, values and draws alike."""
+    st = R.init_state(11, "reference")
+    x, legal = gen_boards(1000, 200, 77)
+    model = make_model(cuda, st, prec)
+    xd, ld = x.to(cuda), legal.to(cuda)
+    u = torch.rand(1000, generator=torch.Generator().manual_seed(5)).to(cuda)
+    with torch.inference_mode():
+        lg, vg = model.forward_masked(xd, ld)
+        ag, pg, _ = model.selfplay_step(xd, u, 0.8, legal=ld)
+        lo, vo = R.forward(st, x)
+        for n in (1, 3, 255, 257, 513, 999):
+            l, v = model.forward_masked(xd[:n], ld[:n])
+            assert torch.equal(l, lg[:n]) and torch.equal(v, vg[:n]), n
+            a, p, _ = model.selfplay_step(xd[:n], u[:n], 0.8, legal=ld[:n])
+            assert torch.equal(a, ag[:n]) and torch.equal(p, pg[:n]), n
+    assert rel_l2(lg.float().cpu().masked_fill(~legal, 0), lo.masked_fill(~legal, 0)) <= BF16_TOL
+    assert rel_l2(vg.float().cpu(), vo) <= BF16_TOL
+
+
 def test_empty_batch(cuda):
     model = c6.PolicyValueNet().to(cuda)
     with torch.inference_mode():
