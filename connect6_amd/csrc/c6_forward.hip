@@ -1126,12 +1126,12 @@ __device__ __forceinline__ void conv3_seg(const unsigned char *smem, const WFrag
 //     epilogue of this layer's own tile 0, which is final after part A.
 // So only single-tile layers convert anything with the matrix pipe idle, and a layer with
 // several cout tiles hands `acc` on with tile 0 already stored.
-template <class P, int L, class Rezero>
+template <class P, int L, class Rezero, class LastHidden>
 __device__ __forceinline__ void pipe_layer(
     unsigned char *smem, const unsigned char *packed, int tail_lds,
     v4i (&ring)[kRing * (kCoutArr[L] / 32)], const int (&ci)[3], int h, int lane, int wave,
     bool trace_on, const int (&lo_scale_w)[8], const f32x16 (&prev)[kCinArr[L] / 32][3],
-    f32x16 (&acc)[kCoutArr[L] / 32][3], Rezero rezero) {
+    f32x16 (&acc)[kCoutArr[L] / 32][3], Rezero rezero, LastHidden last_hidden) {
   using G = Geo<P>;
   constexpr int NT = kCoutArr[L] / 32, NTP = kCinArr[L] / 32;
   constexpr int RIN = act_rot(L), ROUT = act_rot(L + 1);
@@ -1193,7 +1193,11 @@ __device__ __forceinline__ void pipe_layer(
     conv3_seg<P, L, kSegA, NTP - 1>(smem, wl, ring, bq, rb, acc, bias, [](int) {});
     using Plan = EpiPlan<P, Whole, true, kPhaseSteps * (NT - 1) * 3 - 8>;
     conv3_seg<P, L, kSegB, NTP - 1>(smem, wl, ring, bq, rb, acc, bias, [&](int g) __attribute__((always_inline)) {
-      if constexpr (!kLast) Plan::template run<NT>(smem, wb, h4, acc, 0, ROUT, g, carry, k);
+      if constexpr (!kLast) {
+        Plan::template run<NT>(smem, wb, h4, acc, 0, ROUT, g, carry, k);
+      } else {
+        last_hidden(g);  // (the last layer's tile 0 feeds the heads from the accumulators)
+      }
     });
   }
   C6_MARK(4 + 2 * L);
@@ -1497,21 +1501,70 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
         const v4i z = {0, 0, 0, 0};
         *reinterpret_cast<v4i *>(smem + pos * G::PIXB + w16 * 16) = z;
       }
-    });
+    }, [](int) {});
     preload_flat<kRing * 2>(r3, layer_weights<P, 2>(packed, lane));
     f32x16 a2[2][3];
-    pipe_layer<P, 2>(smem, packed, tail_lds, r3, ci, h, lane, wave, trace_on, lo_scale_w, a1, a2, [] {});
+    pipe_layer<P, 2>(smem, packed, tail_lds, r3, ci, h, lane, wave, trace_on, lo_scale_w, a1, a2, [] {}, [](int) {});
     f32x16 a3[2][3];
-    pipe_layer<P, 3>(smem, packed, tail_lds, r3, ci, h, lane, wave, trace_on, lo_scale_w, a2, a3, [] {});
+    pipe_layer<P, 3>(smem, packed, tail_lds, r3, ci, h, lane, wave, trace_on, lo_scale_w, a2, a3, [] {}, [](int) {});
     f32x16 a4[2][3];
-    pipe_layer<P, 4>(smem, packed, tail_lds, r3, ci, h, lane, wave, trace_on, lo_scale_w, a3, a4, [] {});
+    pipe_layer<P, 4>(smem, packed, tail_lds, r3, ci, h, lane, wave, trace_on, lo_scale_w, a3, a4, [] {}, [](int) {});
     preload_flat<kRing * 3>(r6, layer_weights<P, 5>(packed, lane));
     f32x16 a5[3][3];
-    pipe_layer<P, 5>(smem, packed, tail_lds, r6, ci, h, lane, wave, trace_on, lo_scale_w, a4, a5, [] {});
+    pipe_layer<P, 5>(smem, packed, tail_lds, r6, ci, h, lane, wave, trace_on, lo_scale_w, a4, a5, [] {}, [](int) {});
     f32x16 a6[3][3];
-    pipe_layer<P, 6>(smem, packed, tail_lds, r6, ci, h, lane, wave, trace_on, lo_scale_w, a5, a6, [] {});
+    pipe_layer<P, 6>(smem, packed, tail_lds, r6, ci, h, lane, wave, trace_on, lo_scale_w, a5, a6, [] {}, [](int) {});
     f32x16 acc[3][3];
-    pipe_layer<P, 7>(smem, packed, tail_lds, r6, ci, h, lane, wave, trace_on, lo_scale_w, a6, acc, [] {});
+    // The heads' share of channel tile 0 rides behind the MFMAs of the last layer's other two
+    // tiles (tile 0 is final before them): element e = (quad, pixel tile, channel of the quad)
+    // takes exp2 in slot 2e, 1 + . in slot 2e+1, rcp in slot 2e+2 and x * . with the two
+    // multiply-adds in slot 2e+3 -- three instructions per slot in the mean.
+    float pol[3] = {0.0f, 0.0f, 0.0f}, val0[3] = {0.0f, 0.0f, 0.0f};
+    f32x4 hpw[4], hvw[4];
+    float hden[2];
+    auto head_slot = [&](int g) __attribute__((always_inline)) {
+      constexpr int NE = 48;
+      if (g == 0) {
+        int hb0 = tail_lds + 4 * kBiasTotal + 16 * h;
+        asm volatile("" : "+v"(hb0));
+        const float *w0 = reinterpret_cast<const float *>(smem + hb0);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          hpw[q] = *reinterpret_cast<const f32x4 *>(w0 + 8 * q);
+          hvw[q] = *reinterpret_cast<const f32x4 *>(w0 + kHeadC + 8 * q);
+        }
+      }
+      auto reg_of = [](int e) __attribute__((always_inline)) { return 4 * (e / 12) + e % 4; };
+      auto tile_of = [](int e) __attribute__((always_inline)) { return (e / 4) % 3; };
+      // (each result through an empty asm statement: pure arithmetic whose only use comes behind
+      // the K-loop would otherwise be moved there)
+      if (g % 2 == 0) {
+        const int e = g / 2;
+        if (e < NE) {
+          hden[e % 2] = __builtin_amdgcn_exp2f(acc[0][tile_of(e)][reg_of(e)]);
+          asm volatile("" : "+v"(hden[e % 2]));
+        }
+        if (e - 1 >= 0 && e - 1 < NE) {
+          hden[(e - 1) % 2] = __builtin_amdgcn_rcpf(hden[(e - 1) % 2]);
+          asm volatile("" : "+v"(hden[(e - 1) % 2]));
+        }
+      } else {
+        const int e = g / 2;
+        if (e < NE) {
+          hden[e % 2] = 1.0f + hden[e % 2];
+          asm volatile("" : "+v"(hden[e % 2]));
+        }
+        if (e - 1 >= 0 && e - 1 < NE) {
+          const int d = e - 1, j = tile_of(d);
+          const float a = acc[0][j][reg_of(d)] * hden[d % 2];
+          pol[j] = fmaf(a, hpw[d / 12][d % 4], pol[j]);
+          val0[j] = fmaf(a, hvw[d / 12][d % 4], val0[j]);
+          asm volatile("" : "+v"(pol[j]), "+v"(val0[j]));
+        }
+      }
+    };
+    pipe_layer<P, 7>(smem, packed, tail_lds, r6, ci, h, lane, wave, trace_on, lo_scale_w, a6, acc, [] {},
+                     [&](int g) __attribute__((always_inline)) { head_slot(g); });
 
     // ---- both 1x1 heads straight from the fp32 accumulators of layer 8 ----
     {
@@ -1527,10 +1580,11 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
 #pragma unroll
       for (int j = 0; j < 3; ++j) pix[j] = tile_pixel(th, j, valid[j]);
       if (bn < b_end) preload_ring<L1Pipe<P>::D, 1>(r1, fast1_weights(bn));
-      float pol[3] = {0.0f, 0.0f, 0.0f};
       float vsum = 0.0f;
 #pragma unroll
-      for (int t = 0; t < 3; ++t)
+      for (int j = 0; j < 3; ++j) vsum += valid[j] ? val0[j] : 0.0f;  // (tile 0: done behind the last layer)
+#pragma unroll
+      for (int t = 1; t < 3; ++t)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const f32x4 pw = *reinterpret_cast<const f32x4 *>(pwg + 32 * t + 8 * q);
