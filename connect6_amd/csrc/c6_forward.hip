@@ -1700,6 +1700,8 @@ __global__ __launch_bounds__(256) void fused_forward_kernel(const FwdParams prm)
   float xin[ROUNDS][3];
   unsigned char occin[ROUNDS];
   auto fetch_board = [&](long long b) {
+    int tid = threadIdx.x;  // (opaque per call: the per-square addresses are formed here, not kept)
+    asm volatile("" : "+v"(tid));
     if (prm.x_dtype == C6_DT_BOARD_I8) {
       // environment state in, network planes out (connect6/vector_env.py:196-218 of the
       // reference), seen through D4 view prm.view (connect6/train.py:222-230)
@@ -1901,11 +1903,14 @@ __global__ __launch_bounds__(256) void fused_forward_kernel(const FwdParams prm)
       }
     }
     if (prm.actions != nullptr && wave == 0) {
-      const float it = prm.inv_temperature;
+      float it = prm.inv_temperature;
+      asm volatile("" : "+s"(it));  // (what is derived from it is derived here, not kept)
       int a;
       float lp;
+      int lane_here = lane;  // opaque per board: the entries' LDS addresses are computed here,
+      asm volatile("" : "+v"(lane_here));  // not once per kernel into registers that get spilled
       wave_sample(
-          lane, prm.u[b], it, [&](int i) { return lgt[i]; }, [&](int i) { return occ[i] == 0; },
+          lane_here, prm.u[b], it, [&](int i) { return lgt[i]; }, [&](int i) { return occ[i] == 0; },
           a, lp);
       if (lane == 0) {
         prm.actions[b] = a;
