@@ -580,11 +580,15 @@ __device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
     for (int j = 0; j < 3; ++j) {
       b[j][0] = *reinterpret_cast<const v4i *>(smem + pbase[j] + off);
       if constexpr (P::LO6) {
-        // 12 bytes: the last two data dwords and the scale (a 16-byte read would leave a dead
-        // register that the compiler reuses at once, waiting for the read to land first)
-        typedef int v3i __attribute__((ext_vector_type(3)));
-        const v3i q = *reinterpret_cast<const v3i *>(smem + pbase[j] + off + 16);
-        b[j][1] = v4i{q[0], q[1], q[2], q[2]};  // (register 7 is not read: no constant to move in)
+        // The last two data dwords with an 8-byte read, straight into the operand's registers 4
+        // and 5, and the scale on its own (volatile: the compiler would merge the two into one
+        // 12-byte read again, whose three registers cannot be part of the six-register operand,
+        // and copy two of them; a 16-byte read would leave a dead register that the compiler
+        // reuses at once, waiting for the read to land first).
+        const v2i q = *reinterpret_cast<const v2i *>(smem + pbase[j] + off + 16);
+        typedef const volatile __attribute__((address_space(3))) int *LdsVolatileInt;
+        const int sc = *(LdsVolatileInt)(smem + pbase[j] + off + 24);
+        b[j][1] = v4i{q[0], q[1], sc, sc};
       } else {
         b[j][1] = *reinterpret_cast<const v4i *>(smem + pbase[j] + off + 16);
       }
