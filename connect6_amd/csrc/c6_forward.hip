@@ -746,6 +746,9 @@ __device__ __forceinline__ void load_bias_tiles_lds(f32x16 (&bt)[N], const unsig
   int base = 16 * h;
   asm volatile("" : "+v"(base));
   base += tail_lds + 4 * layer_off;
+  // (opaque again behind the sum: the copy sits beyond the 64 KiB that an LDS instruction's
+  // offset field reaches, and folded into one constant per read it costs an addition per read)
+  asm volatile("" : "+v"(base));
 #pragma unroll
   for (int t = 0; t < N; ++t)
 #pragma unroll
