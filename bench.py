@@ -28,8 +28,12 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per B=4096 launch of the fused kernel: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (one
 # run each), scaled by what the same counters read for a 256 MiB copy (x2.00 and x1.00); the
 # figures and commands are in profiles/fused_forward_<mode>_b4096.md.
-TRAFFIC_BYTES = {"bf16f6": 34.4e6, "bf16f8": 33.9e6, "bf16": 31.2e6}
-HEADLINE = "bf16f6"                      # fastest bf16-MFMA mode that meets the >= 99 % argmax gate
+TRAFFIC_BYTES = {"bf16c": None, "bf16f6": 34.4e6, "bf16": 31.2e6}
+# The cascade: every board with plain bf16 layer boundaries, then the boards whose decision is
+# closer than the rounding noise again with the bf16 + fp6 correction.  The fastest bf16-MFMA
+# mode that meets the >= 99 % argmax gate; its time depends on how many boards go twice, which
+# the line reports.
+HEADLINE = "bf16c"
 
 
 def main() -> int:
@@ -38,7 +42,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--batch", type=int, default=4096)
-    ap.add_argument("--precision", default=HEADLINE, choices=["bf16f6", "bf16f8", "bf16x2", "bf16", "fp16", "fp32"])
+    ap.add_argument("--precision", default=HEADLINE, choices=["bf16c", "bf16f6", "bf16", "fp16", "fp32"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="headline + roofline only")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -91,6 +95,19 @@ def main() -> int:
     wall, kern = run_mode(args.precision, K, W)
     value = B / wall
     achieved = B * CONV_FLOP_PER_BOARD / kern / 1e12
+    kernel_name = {"fp32": "fused_forward_kernel<fp32>"}.get(args.precision, f"fused_pipe_kernel<{args.precision}>")
+    cascade = None
+    if args.precision == "bf16c":
+        # HIP events bracket the whole step: the reset of the list, the bf16 kernel over all
+        # boards, the bf16 + fp6 kernel over the listed ones.  The first pass alone is timed with
+        # threshold 0 (no board listed; the second kernel still starts and finds nothing).
+        kernel_name = "fused_pipe_kernel<bf16> over all boards + fused_pipe_kernel<bf16f6> over the listed boards"
+        twice = int(model.cascade_stats["second_pass"].item())
+        model.cascade_threshold = 0.0
+        _, first = run_mode("bf16c", max(5, K // 2), 3)
+        model.cascade_threshold = None
+        cascade = {"threshold": c6.CASCADE_THRESHOLD, "boards_evaluated_twice": twice, "fraction": twice / B,
+                   "first_pass_ms": first * 1e3, "second_pass_ms": (kern - first) * 1e3}
     out = {
         "metric": "boards/sec B=4096 bf16 forward + % MFMA peak; G=8 grouped-history boards/sec",
         "value": value,
@@ -118,11 +135,13 @@ def main() -> int:
             "frac": achieved / MFMA_PEAK_TFLOPS,
             "traffic": TRAFFIC_BYTES.get(args.precision),
             "traffic_unit": "bytes per launch",
-            "kernel": "fused_pipe_kernel" if args.precision in ("bf16f6", "bf16", "fp16") else "fused_forward_kernel",
+            "kernel": kernel_name,
             "kernel_ms": kern * 1e3,
             "flop_per_board": CONV_FLOP_PER_BOARD,
         },
     }
+    if cascade is not None:
+        out["roofline"]["cascade"] = cascade
     # What this card sustains on back-to-back bf16 MFMAs alone (every CU, one wave per SIMD): the
     # published peak assumes the top shader clock, which the card's power management does not hold
     # under a dense matrix load with ordinary operand bits.  Reported beside the roofline, which
@@ -145,7 +164,7 @@ def main() -> int:
         with torch.inference_mode():
             l32, v32 = model.forward_masked(x, fill=float("-inf"))
         modes = {}
-        for prec in ("bf16f6", "bf16f8", "bf16x2", "bf16", "fp16", "fp32"):
+        for prec in ("bf16c", "bf16f6", "bf16", "fp16", "fp32"):
             w_, k_ = run_mode(prec, max(5, K // 2), 3)
             with torch.inference_mode():
                 lg, vg = model.forward_masked(x, fill=float("-inf"))

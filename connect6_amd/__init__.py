@@ -4,7 +4,7 @@ Host-side mirror of the reference's operator interface for this path
 (connect6/model.py, connect6/history.py:186-303 and connect6/vector_env.py) over
 a C-ABI library of hand-written HIP kernels.
 """
-from ._lib import C6Error, build, load, probe_mfma_rate
+from ._lib import CASCADE_THRESHOLD, C6Error, build, load, probe_mfma_rate
 from .history import HistoricalCheckpoint, HistoricalPolicyEnsemble, history_dtype
 from .model import PolicyValueNet, build_model, mask_logits
 from .selfplay import (
@@ -20,6 +20,7 @@ from .selfplay import (
 from .vector_env import StepBatch, VectorConnect6, canonical_network_input, canonical_observation
 
 __all__ = [
+    "CASCADE_THRESHOLD",
     "C6Error",
     "HistoricalCheckpoint",
     "HistoricalPolicyEnsemble",

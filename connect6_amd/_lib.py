@@ -18,9 +18,12 @@ _SOURCES = ("c6_forward.hip", "c6_tail.hip", "c6_generic.hip", "c6_env.hip", "c6
 _RESOURCES = _LIBDIR / "resource_usage.txt"   # registers, scratch and LDS of every kernel, written by build()
 
 # arithmetic modes (include/connect6_amd.h)
-PREC_F32, PREC_BF16, PREC_F16, PREC_BF16X2, PREC_BF16F8, PREC_BF16F6 = 0, 1, 2, 3, 4, 5
+PREC_F32, PREC_BF16, PREC_F16, PREC_BF16X2, PREC_BF16F8, PREC_BF16F6, PREC_BF16C = 0, 1, 2, 3, 4, 5, 6
 PREC_BY_NAME = {"fp32": PREC_F32, "bf16": PREC_BF16, "fp16": PREC_F16, "bf16x2": PREC_BF16X2,
-                "bf16f8": PREC_BF16F8, "bf16f6": PREC_BF16F6}
+                "bf16f8": PREC_BF16F8, "bf16f6": PREC_BF16F6, "bf16c": PREC_BF16C}
+# cascade mode: a board is evaluated a second time (corrected arithmetic) when its best free
+# square leads the second best by less than this many standard deviations of its logits
+CASCADE_THRESHOLD = 0.03
 DT_F32, DT_BF16, DT_F16 = 0, 1, 2
 MASK_NONE, MASK_INPUT, MASK_LEGAL = 0, 1, 2
 
@@ -32,6 +35,9 @@ EXPORTS = (
     "c6_pack_weights",
     "c6_forward",
     "c6_forward_boards",
+    "c6_cascade_workspace_bytes",
+    "c6_forward_cascade",
+    "c6_forward_boards_cascade",
     "c6_generic_workspace_bytes",
     "c6_forward_generic",
     "c6_forward_generic_static",
@@ -156,6 +162,14 @@ def load() -> ctypes.CDLL:
     lib.c6_forward_boards.restype = i32
     lib.c6_forward_boards.argtypes = [vp, vp, vp, i64, vp, i32, i64, vp, i32, vp, vp, i32, f32, vp, f32,
                                       vp, vp, vp]
+    lib.c6_cascade_workspace_bytes.restype = i32
+    lib.c6_cascade_workspace_bytes.argtypes = [i64, ctypes.POINTER(ctypes.c_size_t)]
+    lib.c6_forward_cascade.restype = i32
+    lib.c6_forward_cascade.argtypes = [vp, i32, i64, i64, vp, ctypes.c_size_t, vp, vp, i32, vp, f32,
+                                       vp, f32, vp, vp, f32, vp, ctypes.c_size_t, vp]
+    lib.c6_forward_boards_cascade.restype = i32
+    lib.c6_forward_boards_cascade.argtypes = [vp, vp, vp, i64, vp, i32, i64, vp, vp, vp, i32, f32, vp, f32,
+                                              vp, vp, f32, vp, ctypes.c_size_t, vp]
     ip = ctypes.POINTER(ctypes.c_int)
     lib.c6_generic_workspace_bytes.restype = i32
     lib.c6_generic_workspace_bytes.argtypes = [i64, i32, i32, ip, ctypes.POINTER(ctypes.c_size_t)]
@@ -198,6 +212,12 @@ def check(rc: int, what: str) -> None:
 def packed_bytes(prec: int) -> int:
     n = ctypes.c_size_t(0)
     check(load().c6_packed_bytes(prec, ctypes.byref(n)), "c6_packed_bytes")
+    return int(n.value)
+
+
+def cascade_workspace_bytes(boards: int) -> int:
+    n = ctypes.c_size_t(0)
+    check(load().c6_cascade_workspace_bytes(int(boards), ctypes.byref(n)), "c6_cascade_workspace_bytes")
     return int(n.value)
 
 

@@ -19,6 +19,7 @@ void set_error(const char *fmt, ...) {
 
 int dispatch_pack(int prec, const PackParams &pp, hipStream_t st);
 int dispatch_forward(int prec, const FwdParams &fp, hipStream_t st);
+int dispatch_cascade(const FwdParams &fp, float threshold, void *workspace, hipStream_t st);
 size_t packed_bytes(int prec);
 int launch_mask(const void *, const uint8_t *, int, long long, uint32_t, void *, hipStream_t);
 int launch_sample(const float *, const uint8_t *, const float *, float, long long, long long *,
@@ -77,7 +78,17 @@ static int device_ok(const char *who) {
 
 static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 static int elem_bytes(int dt) { return dt == C6_DT_F32 ? 4 : ((dt == C6_DT_BF16 || dt == C6_DT_F16) ? 2 : 0); }
-static bool valid_prec(int p) { return p >= C6_PREC_F32 && p <= C6_PREC_BF16F6; }
+static bool valid_prec(int p) { return p >= C6_PREC_F32 && p <= C6_PREC_BF16C; }
+
+// the cascade's workspace argument, checked; `who` names the entry point in the message
+static int check_cascade_workspace(const char *who, long long boards, const void *workspace, size_t bytes) {
+  if (workspace == nullptr || !aligned16(workspace) || bytes < cascade_workspace_bytes(boards)) {
+    set_error("%s: the workspace must be a 16-byte aligned device buffer of at least %zu bytes "
+              "(c6_cascade_workspace_bytes), got %zu", who, cascade_workspace_bytes(boards), bytes);
+    return C6_EINVAL;
+  }
+  return C6_OK;
+}
 
 }  // namespace c6
 
@@ -131,45 +142,49 @@ int c6_pack_weights(const float *const *conv_w, const float *const *conv_b, cons
   return dispatch_pack(prec, pp, static_cast<hipStream_t>(stream));
 }
 
-int c6_forward(const void *x, int x_dtype, int64_t groups, int64_t boards_per_group,
-               const void *packed, size_t packed_stride, int prec, float *logits, float *value,
-               int mask_mode, const uint8_t *legal, float fill, const float *u, float temperature,
-               int64_t *actions, float *logprob, void *stream) {
-  if (!valid_prec(prec)) {
-    set_error("c6_forward: unknown precision mode %d", prec);
+// c6_forward and c6_forward_cascade (workspace != nullptr: the latter)
+static int forward_planes(const char *who, const void *x, int x_dtype, int64_t groups,
+                          int64_t boards_per_group, const void *packed, size_t packed_stride,
+                          int prec, float *logits, float *value, int mask_mode,
+                          const uint8_t *legal, float fill, const float *u, float temperature,
+                          int64_t *actions, float *logprob, bool cascade, float threshold,
+                          void *workspace, size_t workspace_bytes, void *stream) {
+  if (!valid_prec(prec) || (prec == C6_PREC_BF16C) != cascade) {
+    set_error("%s: precision mode %d is unknown or not served by this entry point (C6_PREC_BF16C "
+              "takes c6_forward_cascade, every other mode c6_forward)", who, prec);
     return C6_EINVAL;
   }
   if (elem_bytes(x_dtype) == 0) {
-    set_error("c6_forward: unknown input element type %d", x_dtype);
+    set_error("%s: unknown input element type %d", who, x_dtype);
     return C6_EINVAL;
   }
   if (groups < 1 || boards_per_group < 0) {
-    set_error("c6_forward: groups=%lld boards_per_group=%lld out of range", (long long)groups,
+    set_error("%s: groups=%lld boards_per_group=%lld out of range", who, (long long)groups,
               (long long)boards_per_group);
     return C6_EINVAL;
   }
   if (boards_per_group == 0) return C6_OK;  // empty batch: nothing to do
   if (groups > 0x7fffffffLL / boards_per_group) {
-    set_error("c6_forward: %lld x %lld boards exceed the 2^31-1 boards one launch can index",
+    set_error("%s: %lld x %lld boards exceed the 2^31-1 boards one launch can index", who,
               (long long)groups, (long long)boards_per_group);
     return C6_EINVAL;
   }
   if (x == nullptr || packed == nullptr) {
-    set_error("c6_forward: x and packed must not be null");
+    set_error("%s: x and packed must not be null", who);
     return C6_EINVAL;
   }
   if (!aligned16(packed) || (packed_stride & 15u) != 0 ||
       (groups > 1 && packed_stride < packed_bytes(prec))) {
-    set_error("c6_forward: packed weights must be 16-byte aligned with stride >= one set");
+    set_error("%s: packed weights must be 16-byte aligned with stride >= one set", who);
     return C6_EINVAL;
   }
   if (mask_mode < C6_MASK_NONE || mask_mode > C6_MASK_LEGAL ||
       (mask_mode == C6_MASK_LEGAL && legal == nullptr)) {
-    set_error("c6_forward: bad mask_mode %d (legal mask %s)", mask_mode, legal ? "given" : "missing");
+    set_error("%s: bad mask_mode %d (legal mask %s)", who, mask_mode, legal ? "given" : "missing");
     return C6_EINVAL;
   }
   if (actions != nullptr && u == nullptr) {
-    set_error("c6_forward: sampling needs the uniform draws u");
+    set_error("%s: sampling needs the uniform draws u", who);
     return C6_EINVAL;
   }
   FwdParams fp;
@@ -193,40 +208,75 @@ int c6_forward(const void *x, int x_dtype, int64_t groups, int64_t boards_per_gr
   fp.index = nullptr;
   fp.num_states = 0;
   fp.view = 0;
-  C6_REQUIRE_DEVICE("c6_forward");
+  if (cascade) {
+    const int rc = check_cascade_workspace(who, fp.total_boards, workspace, workspace_bytes);
+    if (rc != C6_OK) return rc;
+  }
+  C6_REQUIRE_DEVICE(who);
+  if (cascade) return dispatch_cascade(fp, threshold, workspace, static_cast<hipStream_t>(stream));
   return dispatch_forward(prec, fp, static_cast<hipStream_t>(stream));
 }
 
-int c6_forward_boards(const int8_t *boards, const int8_t *player, const int8_t *stones_left,
-                      int64_t num_states, const int64_t *index, int view, int64_t batch,
-                      const void *packed, int prec,
-                      float *logits, float *value, int mask_mode, float fill, const float *u,
-                      float temperature, int64_t *actions, float *logprob, void *stream) {
-  if (!valid_prec(prec) || batch < 0 || batch > 0x7fffffffLL || view < 0 || view > 7 || num_states < 0) {
-    set_error("c6_forward_boards: bad precision %d, batch %lld, states %lld or view %d", prec,
+int c6_forward(const void *x, int x_dtype, int64_t groups, int64_t boards_per_group,
+               const void *packed, size_t packed_stride, int prec, float *logits, float *value,
+               int mask_mode, const uint8_t *legal, float fill, const float *u, float temperature,
+               int64_t *actions, float *logprob, void *stream) {
+  return forward_planes("c6_forward", x, x_dtype, groups, boards_per_group, packed, packed_stride, prec,
+                        logits, value, mask_mode, legal, fill, u, temperature, actions, logprob, false,
+                        0.0f, nullptr, 0, stream);
+}
+
+int c6_cascade_workspace_bytes(int64_t boards, size_t *bytes) {
+  if (boards < 0 || boards > 0x7fffffffLL || bytes == nullptr) {
+    set_error("c6_cascade_workspace_bytes: board count out of range or null output");
+    return C6_EINVAL;
+  }
+  *bytes = cascade_workspace_bytes(boards);
+  return C6_OK;
+}
+
+int c6_forward_cascade(const void *x, int x_dtype, int64_t groups, int64_t boards_per_group,
+                       const void *packed, size_t packed_stride, float *logits, float *value,
+                       int mask_mode, const uint8_t *legal, float fill, const float *u,
+                       float temperature, int64_t *actions, float *logprob, float threshold,
+                       void *workspace, size_t workspace_bytes, void *stream) {
+  return forward_planes("c6_forward_cascade", x, x_dtype, groups, boards_per_group, packed, packed_stride,
+                        C6_PREC_BF16C, logits, value, mask_mode, legal, fill, u, temperature, actions,
+                        logprob, true, threshold, workspace, workspace_bytes, stream);
+}
+
+
+static int forward_states(const char *who, const int8_t *boards, const int8_t *player,
+                          const int8_t *stones_left, int64_t num_states, const int64_t *index,
+                          int view, int64_t batch, const void *packed, int prec, float *logits,
+                          float *value, int mask_mode, float fill, const float *u,
+                          float temperature, int64_t *actions, float *logprob, bool cascade,
+                          float threshold, void *workspace, size_t workspace_bytes, void *stream) {
+  if (!valid_prec(prec) || (prec == C6_PREC_BF16C) != cascade || batch < 0 || batch > 0x7fffffffLL || view < 0 || view > 7 || num_states < 0) {
+    set_error("%s: bad precision %d, batch %lld, states %lld or view %d", who, prec,
               (long long)batch, (long long)num_states, view);
     return C6_EINVAL;
   }
   if (batch == 0) return C6_OK;
   if (num_states < 1 || (index == nullptr && batch > num_states)) {
-    set_error("c6_forward_boards: %lld boards requested from %lld states", (long long)batch,
+    set_error("%s: %lld boards requested from %lld states", who, (long long)batch,
               (long long)num_states);
     return C6_EINVAL;
   }
   if (boards == nullptr || player == nullptr || stones_left == nullptr || packed == nullptr) {
-    set_error("c6_forward_boards: boards, player, stones_left and packed must not be null");
+    set_error("%s: boards, player, stones_left and packed must not be null", who);
     return C6_EINVAL;
   }
   if (!aligned16(packed)) {
-    set_error("c6_forward_boards: packed weights must be 16-byte aligned");
+    set_error("%s: packed weights must be 16-byte aligned", who);
     return C6_EINVAL;
   }
   if (mask_mode != C6_MASK_NONE && mask_mode != C6_MASK_INPUT) {
-    set_error("c6_forward_boards: mask_mode must be C6_MASK_NONE or C6_MASK_INPUT, got %d", mask_mode);
+    set_error("%s: mask_mode must be C6_MASK_NONE or C6_MASK_INPUT, got %d", who, mask_mode);
     return C6_EINVAL;
   }
   if (actions != nullptr && u == nullptr) {
-    set_error("c6_forward_boards: sampling needs the uniform draws u");
+    set_error("%s: sampling needs the uniform draws u", who);
     return C6_EINVAL;
   }
   FwdParams fp;
@@ -250,9 +300,37 @@ int c6_forward_boards(const int8_t *boards, const int8_t *player, const int8_t *
   fp.index = reinterpret_cast<const long long *>(index);
   fp.num_states = num_states;
   fp.view = view;
-  C6_REQUIRE_DEVICE("c6_forward_boards");
+  if (cascade) {
+    const int rc = check_cascade_workspace(who, batch, workspace, workspace_bytes);
+    if (rc != C6_OK) return rc;
+  }
+  C6_REQUIRE_DEVICE(who);
+  if (cascade) return dispatch_cascade(fp, threshold, workspace, static_cast<hipStream_t>(stream));
   return dispatch_forward(prec, fp, static_cast<hipStream_t>(stream));
 }
+
+int c6_forward_boards(const int8_t *boards, const int8_t *player, const int8_t *stones_left,
+                      int64_t num_states, const int64_t *index, int view, int64_t batch,
+                      const void *packed, int prec,
+                      float *logits, float *value, int mask_mode, float fill, const float *u,
+                      float temperature, int64_t *actions, float *logprob, void *stream) {
+  return forward_states("c6_forward_boards", boards, player, stones_left, num_states, index, view, batch,
+                        packed, prec, logits, value, mask_mode, fill, u, temperature, actions, logprob,
+                        false, 0.0f, nullptr, 0, stream);
+}
+
+int c6_forward_boards_cascade(const int8_t *boards, const int8_t *player,
+                              const int8_t *stones_left, int64_t num_states,
+                              const int64_t *index, int view, int64_t batch, const void *packed,
+                              float *logits, float *value, int mask_mode, float fill,
+                              const float *u, float temperature, int64_t *actions,
+                              float *logprob, float threshold, void *workspace,
+                              size_t workspace_bytes, void *stream) {
+  return forward_states("c6_forward_boards_cascade", boards, player, stones_left, num_states, index, view,
+                        batch, packed, C6_PREC_BF16C, logits, value, mask_mode, fill, u, temperature,
+                        actions, logprob, true, threshold, workspace, workspace_bytes, stream);
+}
+
 
 static int check_arch(const char *who, int board, int layers, const int *kernels,
                       const int *channels) {

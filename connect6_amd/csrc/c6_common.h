@@ -63,6 +63,7 @@ struct PrecF32 {
   static constexpr int LO8 = 0;
   static constexpr int LO6 = 0;
   static constexpr int LO_FIRST = 1;  // first layer (0-based) whose input carries a low-order part
+  static constexpr int LO_MASK = 0xfe; // pipelined kernel: bit l set = layer l (0-based) runs a low-order pass
 };
 struct PrecBF16 {
   static constexpr int PIPE = 1;      // runs the pipelined kernel (weights packed phase-major)
@@ -72,6 +73,7 @@ struct PrecBF16 {
   static constexpr int LO8 = 0;
   static constexpr int LO6 = 0;
   static constexpr int LO_FIRST = 1;  // first layer (0-based) whose input carries a low-order part
+  static constexpr int LO_MASK = 0xfe; // pipelined kernel: bit l set = layer l (0-based) runs a low-order pass
 };
 struct PrecF16 {
   static constexpr int PIPE = 1;      // runs the pipelined kernel (weights packed phase-major)
@@ -81,6 +83,7 @@ struct PrecF16 {
   static constexpr int LO8 = 0;
   static constexpr int LO6 = 0;
   static constexpr int LO_FIRST = 1;  // first layer (0-based) whose input carries a low-order part
+  static constexpr int LO_MASK = 0xfe; // pipelined kernel: bit l set = layer l (0-based) runs a low-order pass
 };
 struct PrecBF16X2 {
   static constexpr int PIPE = 0;      // runs the layer-by-layer kernel
@@ -90,6 +93,7 @@ struct PrecBF16X2 {
   static constexpr int LO8 = 0;
   static constexpr int LO6 = 0;
   static constexpr int LO_FIRST = 1;  // first layer (0-based) whose input carries a low-order part
+  static constexpr int LO_MASK = 0xfe; // pipelined kernel: bit l set = layer l (0-based) runs a low-order pass
 };
 struct PrecBF16F8 {
   static constexpr int PIPE = 0;      // runs the layer-by-layer kernel
@@ -99,6 +103,7 @@ struct PrecBF16F8 {
   static constexpr int LO8 = 1;       // bf16 plane + the dropped low-order part as scaled fp8
   static constexpr int LO6 = 0;
   static constexpr int LO_FIRST = 1;  // first layer (0-based) whose input carries a low-order part
+  static constexpr int LO_MASK = 0xfe; // pipelined kernel: bit l set = layer l (0-based) runs a low-order pass
 };
 struct PrecBF16F6 {
   static constexpr int PIPE = 1;      // runs the pipelined kernel (weights packed phase-major)
@@ -112,6 +117,10 @@ struct PrecBF16F6 {
   // at B=4096 the mean / worst agreement is 99.23 / 99.10 % with all layers, 99.13 / 99.00 % from
   // layer 4 on, 98.97 / 98.85 % from layer 5 on, 98.85 / 98.58 % from layer 6 on.
   static constexpr int LO_FIRST = 1;
+#ifndef C6_LO_MASK
+#define C6_LO_MASK 0xfe
+#endif
+  static constexpr int LO_MASK = C6_LO_MASK;  // bit l set = layer l (0-based) runs a low-order pass
 };
 
 // bf16 + fp8 mode: what rounding an activation to bf16 drops (|lo| <= 2^-9 |a|) is kept as
@@ -214,11 +223,20 @@ template <class P> struct Geo {
   static constexpr size_t PACKED_BYTES = TAIL_OFF + (size_t)TAIL_FLOATS * 4;
 };
 
+// Cascade mode (C6_PREC_BF16C): one packed set = the plain bf16 set, then (256-byte aligned)
+// the bf16 + fp6 set of the same parameters.
+constexpr size_t kCascadeSecondOffset = (Geo<PrecBF16>::PACKED_BYTES + 255) & ~(size_t)255;
+constexpr size_t kCascadePackedBytes = kCascadeSecondOffset + Geo<PrecBF16F6>::PACKED_BYTES;
+// its workspace: int32 count (+ 3 words of padding), then one int32 per board
+constexpr size_t cascade_workspace_bytes(long long boards) { return (size_t)(16 + 4 * boards + 15) & ~(size_t)15; }
+
 constexpr int bias_offset(int l) {
   int s = 0;
   for (int i = 0; i < l; ++i) s += kCoutArr[i];
   return s;
 }
+
+enum : int { kRedoNone = 0, kRedoDetect = 1, kRedoConsume = 2 };
 
 struct FwdParams {
   const void *x;
@@ -242,6 +260,11 @@ struct FwdParams {
   const long long *index;     // [B] rows of the state tensors to evaluate, or null for 0..B-1
   long long num_states;       // N: index entries are clamped into [0, N) (no out-of-bounds read)
   int view;                   // D4 view 0..7 applied to the board before evaluation
+  // cascade (C6_PREC_BF16C; pipelined kernel only)
+  int redo_mode = kRedoNone;      // kRedoDetect: first pass, kRedoConsume: second pass
+  float redo_threshold = 0.0f;    // first pass: < 0 = every board goes on the list
+  int *redo_count = nullptr;      // number of list entries (device memory)
+  int *redo_list = nullptr;       // boards for the second pass (device memory, one int per board)
 };
 
 struct PackParams {

@@ -67,6 +67,59 @@ __device__ __forceinline__ float wave_inclusive_sum(float v) {
   return v;
 }
 
+__device__ __forceinline__ float wave_min(float v) {
+  return __builtin_bit_cast(float, wave_allreduce_bits(__builtin_bit_cast(int, v), [](int a, int b) {
+    return __builtin_bit_cast(int, fminf(__builtin_bit_cast(float, a), __builtin_bit_cast(float, b)));
+  }));
+}
+
+// Does the largest of a board's 361 logits (entries with ok(i) only) lead the second largest by
+// less than `tau` standard deviations of those logits?  One wave; tau < 0 answers yes for every
+// board, and a board with fewer than two such entries has no margin to judge: no.
+// Everything is taken relative to the largest logit, so a large common offset of the logits
+// (flat policies) costs no precision.
+template <class FZ, class FOK>
+__device__ __forceinline__ bool wave_margin_below(int lane, float tau, FZ z, FOK ok) {
+  constexpr int PER = 6;  // 64 lanes x 6 = 384 >= 361
+  float v[PER];
+  float m = -INFINITY;
+  int n = 0;
+#pragma unroll
+  for (int e = 0; e < PER; ++e) {
+    const int i = lane * PER + e;
+    const bool use = (i < kPix) && ok(i);
+    v[e] = use ? z(i) : -INFINITY;
+    m = fmaxf(m, v[e]);
+    n += use ? 1 : 0;
+  }
+  m = wave_max(m);
+  // d = largest - logit >= 0: the margin is the second smallest d (the smallest is 0)
+  float d1 = INFINITY, d2 = INFINITY, s = 0.0f, ss = 0.0f;
+#pragma unroll
+  for (int e = 0; e < PER; ++e) {
+    if (v[e] != -INFINITY) {
+      const float d = m - v[e];
+      s += d;
+      ss = fmaf(d, d, ss);
+      d2 = d < d1 ? d1 : fminf(d2, d);
+      d1 = fminf(d1, d);
+    }
+  }
+  const float cnt = wave_sum((float)n);
+  s = wave_sum(s);
+  ss = wave_sum(ss);
+  // one lane that holds a largest logit answers with its second smallest d, every other lane
+  // with its smallest (a second lane with a largest logit answers 0: a tie)
+  const unsigned long long tops = __builtin_amdgcn_ballot_w64(d1 == 0.0f);
+  const int owner = tops != 0 ? __builtin_ctzll(tops) : 0;
+  const float gap = wave_min(lane == owner ? d2 : d1);
+  if (cnt < 2.0f) return false;
+  if (tau < 0.0f) return true;
+  const float mean = s / cnt;
+  const float var = fmaxf(ss / cnt - mean * mean, 0.0f);
+  return gap * gap < tau * tau * var;
+}
+
 // Masked softmax + inverse-CDF draw over 361 entries by ONE wave.
 // z(i) must return the logit of entry i, ok(i) its legality; inv_t = 1 / temperature.
 // action = first i with running sum of exp(z/T - max) > u * total, clamped to the last legal

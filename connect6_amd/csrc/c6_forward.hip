@@ -233,8 +233,10 @@ struct WFrags {
   __device__ __forceinline__ v4i operator[](int f) const {
     return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_off, base + f * 1024, 0));
   }
-  __device__ __forceinline__ v2i first8(int f) const {  // the first 8 of the lane's 16 bytes
-    return __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(rsrc, lane_off, base + f * 1024, 0));
+  // 8 bytes per lane of a fragment whose lanes lie 8 bytes apart (the fragment's first 512 bytes):
+  // the load then touches 8 of the L1's 64-byte sectors instead of 16 half-used ones
+  __device__ __forceinline__ v2i dense8(int f) const {
+    return __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(rsrc, lane_off >> 1, base + f * 1024, 0));
   }
   __device__ __forceinline__ WFrags operator+(int f) const { return WFrags{rsrc, lane_off, base + f * 1024}; }
 };
@@ -276,10 +278,9 @@ template <int B, int E, class F> __device__ __forceinline__ void static_for(F &&
   }
 }
 
-#ifndef C6_EXP_LOMASK
-#define C6_EXP_LOMASK 0xff  // (tuning builds: which layers run their low-order pass)
+#ifndef C6_X_LO_NUM
+#define C6_X_LO_NUM 8
 #endif
-
 constexpr int kAhead = 2;  // k-steps between the LDS read of an activation fragment and its MFMAs
 
 // Issue order inside one k-step: memory instructions are dealt out one at a time between
@@ -462,7 +463,7 @@ template <class P>
 __device__ __forceinline__ void lo_load_pieces(const WFrags &src, v4i &p0, v4i &p1) {
   p0 = src[0];
   if constexpr (P::LO6) {
-    const v2i q = src.first8(1);
+    const v2i q = src.dense8(1);
     p1 = v4i{q[0], q[1], 0, 0};
   } else {
     p1 = src[1];
@@ -604,7 +605,9 @@ __device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
   auto chunk = [&](int grp, int d, auto first, auto is_static) __attribute__((always_inline)) {
     const WFrags wn = wl + (grp + 1) * (D * NT * 2);
     v4i(&bcur)[3][2] = bq[d % (kAhead + 1)];
+#ifndef C6_X_NOLOA
     fetch(grp + (d + kAhead) / D, (d + kAhead) % D, is_static, bq[(d + kAhead) % (kAhead + 1)]);
+#endif
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       const v8i a = __builtin_shufflevector(ring0[d][t], ring1[d][t], 0, 1, 2, 3, 4, 5, 6, 7);
@@ -625,8 +628,10 @@ __device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
       }
     }
     // weights of chunk c0 + d + D (the tail over-reads the next layer's copy or the zero padding)
+#ifndef C6_X_NOLOW
 #pragma unroll
     for (int t = 0; t < NT; ++t) lo_load_pieces<P>(wn + (d * NT + t) * 2, ring0[d][t], ring1[d][t]);
+#endif
     interleave_step<NT * 3, 2 * 3, 2 * NT>();
     __builtin_amdgcn_sched_barrier(0);
   };
@@ -1009,8 +1014,8 @@ __device__ __forceinline__ void epi_atom(unsigned char *smem, const int (&wb)[3]
 }
 
 // A schedule as a type: the epilogue of channels R over `SLOTS` MFMA slots.
-template <class P, class R, bool FINISH, int SLOTS> struct EpiPlan {
-  static constexpr EpiSched sched = make_sched(R::CNT, P::LO6 != 0, FINISH, SLOTS);
+template <class P, class R, bool LO, bool FINISH, int SLOTS> struct EpiPlan {
+  static constexpr EpiSched sched = make_sched(R::CNT, LO && P::LO6 != 0, FINISH, SLOTS);
   static_assert(sched.slots <= EpiSched::MAXS, "schedule too long");
   // the atoms of slot g
   template <int NT, bool UNDER_MFMA = true>
@@ -1107,7 +1112,7 @@ __device__ __forceinline__ void conv3_seg(const unsigned char *smem, const WFrag
     constexpr int u = g / (NTS * 3), ti = (g / 3) % NTS, t = T0 + ti, j = g % 3;
     constexpr int f = F0 + u * NTS + ti;
     // (a layer with one input tile runs its low-order pass first, and that one starts from the bias)
-    constexpr bool kLoFirst = P::LO8 && ((C6_EXP_LOMASK >> L) & 1) && NTP == 1;
+    constexpr bool kLoFirst = P::LO8 && ((P::LO_MASK >> L) & 1) && NTP == 1;
     if constexpr (PH == 0 && u == 0 && !kLoFirst) {
       f32x16 c0 = bias[t];
       mma<P>(ring[f % RN], bq[(KS0 + u) % QN][j], c0);
@@ -1159,7 +1164,8 @@ __device__ __forceinline__ void pipe_layer(
   using Whole = EpiRange<0, 16>;
   // (the low-order weight ring is filled in front of the barrier that precedes its pass; filling
   // it a whole phase earlier costs that phase what the pass gains)
-  constexpr bool kLoPass = P::LO8 && ((C6_EXP_LOMASK >> L) & 1);
+  constexpr bool kLoPass = P::LO8 && ((P::LO_MASK >> L) & 1);
+  constexpr bool kLoNext = P::LO8 && L + 1 < kLayers && ((P::LO_MASK >> (L + 1)) & 1);  // this layer's output needs its low-order part
   v4i lor0[LoRing<P, L>::D][LoRing<P, L>::NT], lor1[LoRing<P, L>::D][LoRing<P, L>::NT];
   __syncthreads();  // every wave has finished layer L-1 (its reads, and tile 0 if it stored it there)
   if constexpr (NTP == 1) {
@@ -1167,9 +1173,11 @@ __device__ __forceinline__ void pipe_layer(
     // (a compile-time loop: `#pragma unroll` gives up on a body this size, and a runtime index
     // would put the accumulators into scratch memory)
     rezero();
-    EpiPlan<P, Whole, true, EpiSched::MAXS>::template run_all<NTP>(smem, wb, h4, prev, 0, RIN, carry, k);
-    load_bias_tiles_lds(bias, smem, tail_lds, bias_offset(L), h);
+    // (the low-order ring is asked for in front of the open epilogue, whose arithmetic covers the
+    // round trip to L2)
     if constexpr (kLoPass) lo_preload<P, L>(lor0, lor1, packed, lane);
+    EpiPlan<P, Whole, kLoPass, true, EpiSched::MAXS>::template run_all<NTP>(smem, wb, h4, prev, 0, RIN, carry, k);
+    load_bias_tiles_lds(bias, smem, tail_lds, bias_offset(L), h);
     __syncthreads();
   } else {
     load_bias_tiles_lds(bias, smem, tail_lds, bias_offset(L), h);
@@ -1180,11 +1188,24 @@ __device__ __forceinline__ void pipe_layer(
   // phases 0 .. NTP-2 carry tiles 1 .. NTP-1 of layer L-1
   static_for<0, NTP - 1>([&](auto pc) __attribute__((always_inline)) {
     constexpr int p = decltype(pc)::value;
-    using Plan = EpiPlan<P, Whole, true, kPhaseSteps * NT * 3 - 8>;
+    using Plan = EpiPlan<P, Whole, kLoPass, true, kPhaseSteps * NT * 3 - 8>;
+    // The last of these phases also asks for the low-order pass's first weights, one ring slot
+    // every few MFMAs over its second half: in one burst in front of the barrier the pass starts
+    // by waiting a round trip to L2, and in one burst earlier the loads hold up the phase's own
+    // fragments (the vector memory counter is served in order).
+    constexpr int SLOTS = kPhaseSteps * NT * 3, NLOAD = LoRing<P, L>::D * NT;
+    constexpr int LO_G0 = SLOTS * (C6_X_LO_NUM < 8 ? C6_X_LO_NUM : 0) / 8, LO_STRIDE = (SLOTS - 12 - LO_G0) / NLOAD;
+    static_assert(LO_STRIDE >= 1, "room for the low-order ring loads");
+    const WFrags lo_wl = LoRing<P, L>::base(packed, lane);
     conv3_seg<P, L, kSegFull, p>(smem, wl, ring, bq, rb, acc, bias, [&](int g) __attribute__((always_inline)) {
       Plan::template run<NTP>(smem, wb, h4, prev, p + 1, (RIN + p + 1) % 3, g, carry, k);
+      if constexpr (kLoPass && p == NTP - 2 && C6_X_LO_NUM < 8) {
+        const int i = (g - LO_G0) / LO_STRIDE;
+        if (g >= LO_G0 && (g - LO_G0) % LO_STRIDE == 0 && i < NLOAD)
+          lo_load_pieces<P>(lo_wl + i * 2, lor0[i / NT][i % NT], lor1[i / NT][i % NT]);
+      }
     });
-    if constexpr (kLoPass && p == NTP - 2) lo_preload<P, L>(lor0, lor1, packed, lane);
+    if constexpr (kLoPass && p == NTP - 2 && C6_X_LO_NUM >= 8) lo_preload<P, L>(lor0, lor1, packed, lane);
     __syncthreads();
   });
   C6_MARK(30 + L);
@@ -1198,7 +1219,7 @@ __device__ __forceinline__ void pipe_layer(
     conv3_seg<P, L, kSegFull, NTP - 1>(smem, wl, ring, bq, rb, acc, bias, [](int) {});
   } else {
     conv3_seg<P, L, kSegA, NTP - 1>(smem, wl, ring, bq, rb, acc, bias, [](int) {});
-    using Plan = EpiPlan<P, Whole, true, kPhaseSteps * (NT - 1) * 3 - 8>;
+    using Plan = EpiPlan<P, Whole, kLoNext, true, kPhaseSteps * (NT - 1) * 3 - 8>;
     conv3_seg<P, L, kSegB, NTP - 1>(smem, wl, ring, bq, rb, acc, bias, [&](int g) __attribute__((always_inline)) {
       if constexpr (!kLast) {
         Plan::template run<NT>(smem, wb, h4, acc, 0, ROUT, g, carry, k);
@@ -1250,19 +1271,19 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
   float *red = reinterpret_cast<float *>(smem + G::RED_OFF);
 
   const unsigned per_group = (unsigned)prm.boards_per_group;  // board counts fit 32 bits (host-checked)
-  auto packed_of = [&](long long b) {
-    return prm.packed + (size_t)((unsigned)b / per_group) * prm.packed_stride;
+  auto packed_of = [&](unsigned b) {
+    return prm.packed + (size_t)(b / per_group) * prm.packed_stride;
   };
   // Input of one board, asked for a whole board ahead: loads that write LDS directly, 64
   // consecutive elements per instruction (lane l's element lands in word l behind the
   // instruction's LDS base).  Wave w issues chunks w, w + 4, ...
   typedef const __attribute__((address_space(1))) void *GPtr;
   typedef __attribute__((address_space(3))) void *LPtr;
-  auto board_row = [&](long long b) {  // board-state input: which row of the state tensors
+  auto board_row = [&](unsigned b) {  // board-state input: which row of the state tensors
     long long src = prm.index ? prm.index[b] : b;
     return src < 0 ? 0 : (src >= prm.num_states ? prm.num_states - 1 : src);
   };
-  auto issue_fetch = [&](long long b) {
+  auto issue_fetch = [&](unsigned b) {
     // (lane and wave opaque per call: the chunk addresses are then computed here and not kept,
     // one register pair per chunk, for the whole kernel)
     int ln = lane, wv = wave;
@@ -1326,43 +1347,57 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
                                           : (prm.x_dtype == C6_DT_BF16 ? as_bf16 : as_f16);
       }
     }
-    o = 0;
-    if (prm.mask_mode == C6_MASK_LEGAL) o = aux == 0;
-    if (prm.mask_mode == C6_MASK_INPUT) o = (v[0] != 0.0f) || (v[1] != 0.0f);
+    // bit 0: the square's logit is masked in the output; bit 1: the square counts as occupied
+    // when the margin of the board's decision is judged (cascade), whatever the output mask
+    const unsigned taken = prm.mask_mode == C6_MASK_LEGAL ? (aux == 0) : ((v[0] != 0.0f) || (v[1] != 0.0f));
+    o = (prm.mask_mode != C6_MASK_NONE ? taken : 0u) | (taken << 1);
   };
   // the third plane's value at square 0, and whether square p holds another one
   auto plane2_differs = [&](int p) {
     const unsigned *raw = reinterpret_cast<const unsigned *>(smem + G::NEXT_IN_OFF);
-    return prm.x_dtype != C6_DT_BOARD_I8 && raw[2 * kPix + p] != raw[2 * kPix];
+    // (a 16-bit element arrives in the low half of its word; what the load leaves in the
+    // upper half is not part of the value)
+    const unsigned keep = prm.x_dtype == C6_DT_F32 ? 0xffffffffu : 0xffffu;
+    return prm.x_dtype != C6_DT_BOARD_I8 && ((raw[2 * kPix + p] ^ raw[2 * kPix]) & keep) != 0;
   };
-  auto fast1_weights = [&](long long b) { return packed_frags<P>(packed_of(b), lane, G::FAST1_OFF); };
+  auto fast1_weights = [&](unsigned b) { return packed_frags<P>(packed_of(b), lane, G::FAST1_OFF); };
 
   // Each workgroup takes one contiguous run of boards, and the runs are dealt out so that the
   // workgroups of one XCD (workgroup i runs on XCD i % 8) cover one contiguous eighth of the
   // batch: with several weight sets an XCD's L2 then holds only the sets of its own boards, and
   // consecutive boards of a workgroup mostly reuse the set it has just streamed.
-  const long long per = (prm.total_boards + gridDim.x - 1) / gridDim.x;
+  // Cascade, second pass (prm.redo_mode == kRedoConsume): the boards to evaluate are the entries
+  // of the list the first pass wrote, their number sits in device memory.
+  const bool from_list = prm.redo_mode == kRedoConsume;
+  const unsigned n_items = from_list ? (unsigned)*prm.redo_count : (unsigned)prm.total_boards;
+  auto board_of = [&](unsigned i) { return from_list ? (unsigned)prm.redo_list[i] : i; };
+  const unsigned per = (n_items + gridDim.x - 1) / gridDim.x;
   const unsigned xcds = (gridDim.x % 8 == 0) ? 8 : 1;
-  const long long run = (long long)(blockIdx.x % xcds) * (gridDim.x / xcds) + blockIdx.x / xcds;
-  long long b = run * per;
-  const long long b_end = b + per < prm.total_boards ? b + per : prm.total_boards;
-  if (b >= b_end) return;
-  [[maybe_unused]] const long long b_first = b;
+  const unsigned run = (blockIdx.x % xcds) * (gridDim.x / xcds) + blockIdx.x / xcds;
+  // (board counts fit 31 bits, host-checked; a run beyond the last board starts past n_items)
+  const unsigned long long first_item = (unsigned long long)run * per;
+  if (first_item >= n_items) return;
+  unsigned it = (unsigned)first_item;  // position in the run of boards; `b` below is the board itself
+  const unsigned it_end = n_items - it > per ? it + per : n_items;
+  [[maybe_unused]] const unsigned it_first = it;
   v4i r1[L1Pipe<P>::D][1];
   // (the first layer's weight ring is filled, a board ahead, with the stream for a constant
   // third plane; a board that has none refills it)
+  unsigned b = board_of(it);
   preload_ring<L1Pipe<P>::D, 1>(r1, fast1_weights(b));
   issue_fetch(b);
   if (tid == 0) reinterpret_cast<int *>(red)[8] = 0;  // (the first board's flag, see the staging)
+  const unsigned char *packed_before = nullptr;
 
-  for (; b < b_end; ++b) {
+  for (; it < it_end; ++it) {
     int tidv = tid;  // opaque per board: keeps per-thread staging addresses out of long-lived registers
     asm volatile("" : "+v"(tidv));
     const unsigned char *packed = packed_of(b);
     const float *tail = reinterpret_cast<const float *>(packed + G::TAIL_OFF);
     // the weight set's fp32 tail goes to LDS whenever the set changes (see the staging)
     constexpr int TAILN = kBiasTotal + 2 * kHeadC + 4;
-    const bool new_set = b == b_first || packed != packed_of(b - 1);
+    const bool new_set = packed != packed_before;
+    packed_before = packed;
     const int tail_lds = G::TAIL_LDS_OFF;
     // block-scale exponents of the low-order weight copies (E8M0: 127 - log2 of the copy's scale),
     // fetched here, long before any second pass needs them
@@ -1373,16 +1408,17 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
     }
 
 #if defined(C6_DUMP_POINT)
-    const bool trace_on = (b == b_first + 1);  // second board of this workgroup
+    const bool trace_on = (it == it_first + 1);  // second board of this workgroup
 #elif defined(C6_TRACE)
-    const bool trace_on = (b == b_first + 2);  // third board of this workgroup
+    const bool trace_on = (it == it_first + 2);  // third board of this workgroup
 #else
     const bool trace_on = false;
 #endif
     __builtin_amdgcn_s_waitcnt(0);  // this wave's share of the board's input has landed in LDS
     __syncthreads();  // ... and everybody's; previous board fully written out; LDS is free
     C6_MARK(0);
-    const long long bn = b + 1;
+    const bool has_next = it + 1 < it_end;
+    const unsigned bn = has_next ? board_of(it + 1) : b;
     // The third plane's share of the first layer, should the plane turn out constant: the
     // per-square sums of its weights (register i of pixel tile j = channel 8 (i / 4) + 4 h + i % 4),
     // asked for now so that the loads are long back when the K-loop starts; there they are
@@ -1404,14 +1440,14 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
     // ---- stage the input: zero the shifted copies, then scatter the board ----
     // Does the third plane vary?  Any thread that sees it differ from square 0 raises this board's
     // flag (two flags, used in turn: the other one is cleared for the next board meanwhile).
-    int *plane2_flag = reinterpret_cast<int *>(red) + 8 + (int)((b - b_first) & 1);
+    int *plane2_flag = reinterpret_cast<int *>(red) + 8 + (int)((it - it_first) & 1);
     {
       bool varies = false;
 #pragma unroll
       for (int r = 0; r < ROUNDS; ++r)
         if (tidv + r * THREADS < kPix) varies |= plane2_differs(tidv + r * THREADS);
       if (varies) *plane2_flag = 1;
-      if (tid == 0) reinterpret_cast<int *>(red)[8 + (int)((b - b_first + 1) & 1)] = 0;
+      if (tid == 0) reinterpret_cast<int *>(red)[8 + (int)((it - it_first + 1) & 1)] = 0;
     }
     {
       // (unrolled, one address register and immediate offsets: as a loop the same stores take
@@ -1586,7 +1622,7 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
       asm volatile("" : "+v"(th));  // (computed here, not at the top of the board and kept)
 #pragma unroll
       for (int j = 0; j < 3; ++j) pix[j] = tile_pixel(th, j, valid[j]);
-      if (bn < b_end) preload_ring<L1Pipe<P>::D, 1>(r1, fast1_weights(bn));
+      if (has_next) preload_ring<L1Pipe<P>::D, 1>(r1, fast1_weights(bn));
       float vsum = 0.0f;
 #pragma unroll
       for (int j = 0; j < 3; ++j) vsum += valid[j] ? val0[j] : 0.0f;  // (tile 0: done behind the last layer)
@@ -1627,7 +1663,7 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
       // barrier waits for loads that write LDS) and with no K-loop ahead: the counter of loads in
       // flight is served in order, so in front of a K-loop these loads from HBM would hold up
       // its weight fragments.
-      if (bn < b_end) issue_fetch(bn);
+      if (has_next) issue_fetch(bn);
       if (tid == 0 && prm.value != nullptr) {
         float s = 0.0f;
 #pragma unroll
@@ -1641,25 +1677,38 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
     if (prm.logits != nullptr) {
       for (int p = tidv; p < kPix; p += THREADS) {
         const float v = lgt[p];
-        prm.logits[(size_t)b * kPix + p] = occ[p] ? prm.fill : v;
+        prm.logits[(size_t)b * kPix + p] = (occ[p] & 1) ? prm.fill : v;
       }
     }
     if (prm.actions != nullptr && wave == 0) {
-      float it = prm.inv_temperature;
-      asm volatile("" : "+s"(it));  // (what is derived from it is derived here, not kept)
+      float inv_t = prm.inv_temperature;
+      asm volatile("" : "+s"(inv_t));  // (what is derived from it is derived here, not kept)
       int a;
       float lp;
       int lane_here = lane;  // opaque per board: the entries' LDS addresses are computed here,
       asm volatile("" : "+v"(lane_here));  // not once per kernel into registers that get spilled
       wave_sample(
-          lane_here, prm.u[b], it, [&](int i) { return lgt[i]; }, [&](int i) { return occ[i] == 0; },
+          lane_here, prm.u[b], inv_t, [&](int i) { return lgt[i]; }, [&](int i) { return (occ[i] & 1) == 0; },
           a, lp);
       if (lane == 0) {
         prm.actions[b] = a;
         if (prm.logprob != nullptr) prm.logprob[b] = lp;
       }
     }
+    if (prm.redo_mode == kRedoDetect && wave == 1) {
+      // Cascade, first pass: a board whose best free square leads the second best by less than
+      // the threshold (in standard deviations of its free squares' logits) is put on the list
+      // of boards that the second pass evaluates again with the corrected arithmetic.
+      float tau = prm.redo_threshold;
+      asm volatile("" : "+s"(tau));
+      int lane_here = lane;
+      asm volatile("" : "+v"(lane_here));
+      const bool again = wave_margin_below(
+          lane_here, tau, [&](int i) { return lgt[i]; }, [&](int i) { return (occ[i] & 2) == 0; });
+      if (lane == 0 && again) prm.redo_list[atomicAdd(prm.redo_count, 1)] = (int)b;
+    }
     C6_MARK(20);
+    b = bn;
   }
 }
 
@@ -2033,6 +2082,16 @@ template <class P> __global__ void pack_kernel(const PackParams prm) {
           }
         }
       }
+      if constexpr (P::LO6) {
+        // Second piece of an fp6 fragment: 8 bytes per lane, the lanes' parts packed densely into
+        // the fragment's first 512 bytes (WFrags::dense8); the rest of the fragment is zero.
+        if (frag >= G::HI_FRAGS && frag < G::lo_frag_offset(8) && ((frag - G::HI_FRAGS) & 1)) {
+          unsigned char *fb = prm.packed + (size_t)frag * 1024;
+          *reinterpret_cast<v2i *>(fb + lane * 8) = v2i{o[0], o[1]};
+          *reinterpret_cast<v2i *>(fb + 512 + lane * 8) = v2i{0, 0};
+          return;
+        }
+      }
       *reinterpret_cast<v4i *>(dst) = o;
       return;
     }
@@ -2187,6 +2246,13 @@ template <class P> static int launch_forward(const FwdParams &fp, hipStream_t st
 }
 
 int dispatch_pack(int prec, const PackParams &pp, hipStream_t st) {
+  if (prec == C6_PREC_BF16C) {  // both sets of the cascade
+    const int rc = launch_pack<PrecBF16>(pp, st);
+    if (rc != C6_OK) return rc;
+    PackParams second = pp;
+    second.packed = pp.packed + kCascadeSecondOffset;
+    return launch_pack<PrecBF16F6>(second, st);
+  }
   switch (prec) {
     case C6_PREC_F32: return launch_pack<PrecF32>(pp, st);
     case C6_PREC_BF16: return launch_pack<PrecBF16>(pp, st);
@@ -2200,8 +2266,9 @@ int dispatch_pack(int prec, const PackParams &pp, hipStream_t st) {
 }
 
 int dispatch_forward(int prec, const FwdParams &fp, hipStream_t st) {
-#ifdef C6_ONLY_BF16F6  // (tuning builds: compile one arithmetic mode only)
+#ifdef C6_ONLY_BF16F6  // (tuning builds: compile few arithmetic modes only)
   if (prec == C6_PREC_BF16F6) return launch_forward<PrecBF16F6>(fp, st);
+  if (prec == C6_PREC_BF16) return launch_forward<PrecBF16>(fp, st);
   if (prec == C6_PREC_F32) return launch_forward<PrecF32>(fp, st);
   return C6_EINVAL;
 #else
@@ -2218,7 +2285,34 @@ int dispatch_forward(int prec, const FwdParams &fp, hipStream_t st) {
 #endif
 }
 
+__global__ void cascade_reset_kernel(int *count) {
+  if (threadIdx.x == 0) *count = 0;
+}
+
+// Cascade: every board through the plain bf16 kernel, which lists the boards whose decision
+// margin is below `threshold`; then the listed boards through the bf16 + fp6 kernel, which
+// overwrites their outputs.  Three launches on the caller's stream, no host synchronisation:
+// the second kernel reads the length of the list from device memory.
+int dispatch_cascade(const FwdParams &fp, float threshold, void *workspace, hipStream_t st) {
+  int *count = static_cast<int *>(workspace);
+  hipLaunchKernelGGL(cascade_reset_kernel, dim3(1), dim3(64), 0, st, count);
+  FwdParams first = fp;
+  first.redo_mode = kRedoDetect;
+  first.redo_threshold = threshold;
+  first.redo_count = count;
+  first.redo_list = count + 4;
+  int rc = launch_forward<PrecBF16>(first, st);
+  if (rc != C6_OK) return rc;
+  FwdParams second = fp;
+  second.packed = fp.packed + kCascadeSecondOffset;
+  second.redo_mode = kRedoConsume;
+  second.redo_count = count;
+  second.redo_list = count + 4;
+  return launch_forward<PrecBF16F6>(second, st);
+}
+
 size_t packed_bytes(int prec) {
+  if (prec == C6_PREC_BF16C) return kCascadePackedBytes;
   switch (prec) {
     case C6_PREC_F32: return Geo<PrecF32>::PACKED_BYTES;
     case C6_PREC_BF16: return Geo<PrecBF16>::PACKED_BYTES;

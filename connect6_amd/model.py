@@ -83,9 +83,13 @@ def run_forward(
     u: torch.Tensor | None = None,
     temperature: float = 1.0,
     want_logprob: bool = False,
+    threshold: float | None = None,
+    stats: dict | None = None,
 ):
-    """Launch ``c6_forward``; returns (logits, value, actions, logprob), each
-    None when not requested."""
+    """Launch ``c6_forward`` (``c6_forward_cascade`` for the cascade mode, with ``threshold``
+    and a workspace tensor of its own); returns (logits, value, actions, logprob), each None
+    when not requested.  ``stats``, if given, receives ``second_pass`` for the cascade mode: a
+    one-element int32 device tensor, the number of boards that were evaluated twice."""
     lib = _lib.load()
     dev = x.device
     total = groups * boards_per_group
@@ -114,6 +118,17 @@ def run_forward(
 
     stride = packed.numel() // groups if groups > 1 else packed.numel()
     with torch.cuda.device(dev):
+        if prec == _lib.PREC_BF16C:
+            ws = torch.empty(_lib.cascade_workspace_bytes(total) // 4, dtype=torch.int32, device=dev)
+            rc = lib.c6_forward_cascade(
+                x.data_ptr(), _lib.torch_dtype_code(x.dtype), groups, boards_per_group, packed.data_ptr(),
+                stride, ptr(logits), ptr(value), mask_mode, ptr(legal), fill, ptr(u), float(temperature),
+                ptr(actions), ptr(logprob), float(_lib.CASCADE_THRESHOLD if threshold is None else threshold),
+                ws.data_ptr(), ws.numel() * 4, _lib.stream_ptr(dev))
+            if stats is not None:
+                stats["second_pass"] = ws[:1]
+            _lib.check(rc, "c6_forward_cascade")
+            return logits, value, actions, logprob
         rc = lib.c6_forward(x.data_ptr(), _lib.torch_dtype_code(x.dtype), groups, boards_per_group,
                             packed.data_ptr(), stride, prec, ptr(logits), ptr(value), mask_mode,
                             ptr(legal), fill, ptr(u), float(temperature), ptr(actions),
@@ -271,6 +286,8 @@ class PolicyValueNet(nn.Module):
         self._init_weights()
 
         self.precision: str | None = None
+        self.cascade_threshold: float | None = None   # None: _lib.CASCADE_THRESHOLD
+        self.cascade_stats: dict = {}                 # "second_pass": boards evaluated twice (last call)
         self._packed: dict[int, tuple] = {}
         self._epoch = 0
         self.register_load_state_dict_post_hook(lambda module, _keys: module.refresh_weights())
@@ -379,7 +396,8 @@ class PolicyValueNet(nn.Module):
         prec = self.resolve_precision()
         if not self.is_default_architecture:
             return self._generic(x, prec)
-        logits, value, _, _ = run_forward(x, self.packed_weights(prec), prec, 1, int(x.shape[0]))
+        logits, value, _, _ = run_forward(x, self.packed_weights(prec), prec, 1, int(x.shape[0]),
+                                          threshold=self.cascade_threshold, stats=self.cascade_stats)
         return logits, value
 
     def forward_masked(
@@ -401,6 +419,7 @@ class PolicyValueNet(nn.Module):
         logits, value, _, _ = run_forward(
             x, self.packed_weights(prec), prec, 1, int(x.shape[0]),
             mask_mode=mask_mode, legal=legal, fill=fill,
+            threshold=self.cascade_threshold, stats=self.cascade_stats,
         )
         return logits, value
 
@@ -428,6 +447,7 @@ class PolicyValueNet(nn.Module):
             x, self.packed_weights(prec), prec, 1, int(x.shape[0]), want_logits=return_logits,
             mask_mode=_lib.MASK_INPUT if legal is None else _lib.MASK_LEGAL, legal=legal,
             u=u, temperature=temperature, want_logprob=True,
+            threshold=self.cascade_threshold, stats=self.cascade_stats,
         )
         if return_logits:
             return actions, logprob, value, logits
@@ -537,6 +557,18 @@ def _forward_boards(
         return t.data_ptr() if t is not None else None
 
     with torch.cuda.device(dev):
+        if prec == _lib.PREC_BF16C:
+            ws = torch.empty(_lib.cascade_workspace_bytes(b) // 4, dtype=torch.int32, device=dev)
+            thr = _lib.CASCADE_THRESHOLD if model.cascade_threshold is None else model.cascade_threshold
+            rc = _lib.load().c6_forward_boards_cascade(
+                boards.data_ptr(), current_player.data_ptr(), stones_left.data_ptr(), n, ptr(index),
+                int(view), b, packed.data_ptr(), ptr(logits), value.data_ptr(),
+                _lib.MASK_INPUT if masked else _lib.MASK_NONE,
+                _FILL_LOWEST if fill is None else float(fill), ptr(u), float(temperature),
+                ptr(actions), ptr(logprob), float(thr), ws.data_ptr(), ws.numel() * 4, _lib.stream_ptr(dev))
+            model.cascade_stats["second_pass"] = ws[:1]
+            _lib.check(rc, "c6_forward_boards_cascade")
+            return logits, value, actions, logprob
         rc = _lib.load().c6_forward_boards(
             boards.data_ptr(), current_player.data_ptr(), stones_left.data_ptr(), n, ptr(index),
             int(view), b, packed.data_ptr(), prec, ptr(logits), value.data_ptr(),

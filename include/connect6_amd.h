@@ -40,6 +40,10 @@ extern "C" {
 #define C6_PREC_BF16F6 5 /* the same with the low-order part held as block-scaled fp6 (e2m3,
                             one power-of-two scale per 32 channels), at four times the rate */
 
+#define C6_PREC_BF16C 6  /* cascade: every board in C6_PREC_BF16, then the boards whose decision
+                            is closer than the rounding noise again in C6_PREC_BF16F6; needs a
+                            workspace: c6_forward_cascade / c6_forward_boards_cascade */
+
 /* element types of caller tensors */
 #define C6_DT_F32 0
 #define C6_DT_BF16 1
@@ -113,6 +117,36 @@ int c6_forward_boards(const int8_t *boards, const int8_t *player, const int8_t *
                       int prec, float *logits, float *value, int mask_mode, float fill,
                       const float *u, float temperature, int64_t *actions, float *logprob,
                       void *stream);
+
+/* c6_forward / c6_forward_boards in the cascade mode (C6_PREC_BF16C; `packed` holds sets packed
+ * for that mode).  Replaces the same reference calls as they do (connect6/model.py:96-111,
+ * connect6/history.py:276-303, connect6/train.py:730-748, :791-799).
+ * First every board is evaluated with plain bf16 layer boundaries.  A board is evaluated again,
+ * with the low-order correction of C6_PREC_BF16F6, when its largest logit among the free squares
+ * (free as C6_MASK_LEGAL or the input planes say, whatever mask_mode writes) leads the second
+ * largest by less than `threshold` standard deviations of the free squares' logits: that is
+ * where the rounding of the plain pass can change the move that an argmax picks (reference
+ * callers: connect6/benchmark.py:32,44, connect6/evaluate.py:54, connect6/gui_cnn.py:43).  Its
+ * logits, value and draw replace the first ones.  threshold = 0 evaluates no board twice
+ * (results of C6_PREC_BF16), threshold < 0 every board (results of C6_PREC_BF16F6); 0.03 keeps
+ * the corrected mode's agreement with fp32 on random networks while 3-10 % of the boards are
+ * evaluated twice.  A board's results do not depend on the other boards of the batch.
+ *   workspace  device, c6_cascade_workspace_bytes(boards) bytes, 16-byte aligned; after the
+ *              call its first int32 holds the number of boards that were evaluated twice
+ * Three launches on `stream`, no synchronisation with the host. */
+int c6_cascade_workspace_bytes(int64_t boards, size_t *bytes);
+int c6_forward_cascade(const void *x, int x_dtype, int64_t groups, int64_t boards_per_group,
+                       const void *packed, size_t packed_stride, float *logits, float *value,
+                       int mask_mode, const uint8_t *legal, float fill, const float *u,
+                       float temperature, int64_t *actions, float *logprob, float threshold,
+                       void *workspace, size_t workspace_bytes, void *stream);
+int c6_forward_boards_cascade(const int8_t *boards, const int8_t *player,
+                              const int8_t *stones_left, int64_t num_states,
+                              const int64_t *index, int view, int64_t batch, const void *packed,
+                              float *logits, float *value, int mask_mode, float fill,
+                              const float *u, float temperature, int64_t *actions,
+                              float *logprob, float threshold, void *workspace,
+                              size_t workspace_bytes, void *stream);
 
 /* Forward of ONE weight set for any architecture the reference's PolicyValueNet accepts
  * (connect6/model.py:26-77: any board size, odd kernels, positive channel counts), layer by

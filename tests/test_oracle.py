@@ -276,3 +276,116 @@ def test_oracle_reproduces_committed_golden_vectors():
         assert np.allclose(g[f"{init}_value"], value.numpy(), rtol=1e-5, atol=1e-7)
         a, lp = R.sample_inverse_cdf(logits, legal, torch.from_numpy(g["u"]), 1.0)
         assert np.array_equal(g[f"{init}_actions"], a.numpy())
+
+
+# --------------------------------------------------------------------------
+# oracle/lowprec_ref.py: the bf16 + fp6 contract and the cascade's rule
+# --------------------------------------------------------------------------
+from oracle import lowprec_ref as Q
+
+
+def _e2m3_codes_by_hand():
+    """All 32 non-negative code points from their bit fields, no library involved."""
+    out = []
+    for code in range(32):
+        e, m = code >> 3, code & 7
+        out.append((m / 8.0) if e == 0 else (1.0 + m / 8.0) * (2.0 ** (e - 1)))
+    return out
+
+
+def test_e2m3_grid_is_the_enumerated_format():
+    grid = Q.e2m3_grid().tolist()
+    assert grid == _e2m3_codes_by_hand()
+    assert grid == sorted(grid) and len(set(grid)) == 32
+    assert grid[0] == 0.0 and grid[1] == 0.125 and grid[8] == 1.0 and grid[-1] == 7.5
+
+
+def test_quant_e2m3_is_round_to_nearest_even_with_saturation():
+    grid = _e2m3_codes_by_hand()
+    mids = torch.tensor([(a + b) / 2 for a, b in zip(grid, grid[1:])])   # the ties, exactly representable
+    xs = torch.cat([torch.linspace(-9.0, 9.0, 28801), mids, -mids])
+    got = Q.quant_e2m3(xs)
+    for x, g in zip(xs.tolist(), got.tolist()):
+        a = min(abs(x), 7.5)
+        best = min(abs(a - v) for v in grid)
+        cands = [i for i, v in enumerate(grid) if abs(abs(a - v) - best) < 1e-12]
+        want = grid[cands[0]] if len(cands) == 1 else grid[[i for i in cands if i % 2 == 0][0]]  # tie: even mantissa
+        assert abs(g) == want and (g == 0 or (g > 0) == (x > 0)), (x, g, want)
+    on_grid = torch.tensor(grid + [-v for v in grid])
+    assert torch.equal(Q.quant_e2m3(on_grid), on_grid)               # idempotent
+    assert Q.quant_e2m3(torch.tensor([7.74, 8.0, 1e9, -1e9])).tolist() == [7.5, 7.5, 7.5, -7.5]
+
+
+def test_block_scale_is_the_power_of_two_that_puts_the_largest_in_4_to_8():
+    m = torch.cat([torch.rand(4000).mul(40).sub(20).exp2(), torch.tensor([1.0, 2.0, 0.5, 2.0 ** -20, 3.999999, 4.0])])
+    sc = Q.block_scale(m)
+    assert torch.equal(torch.log2(sc), torch.log2(sc).round())       # powers of two
+    r = m / sc
+    assert bool(((r >= 4.0) & (r < 8.0)).all())
+    for v, s in zip(m.tolist()[-6:], sc.tolist()[-6:]):
+        assert s == 2.0 ** (math.floor(math.log2(v)) - 2)
+    assert float(Q.block_scale(torch.tensor([0.0]))) == 2.0 ** -126  # an all-zero block
+
+
+def test_quant_lo_blocks_error_is_half_a_step_of_the_block_scale():
+    g = torch.Generator().manual_seed(3)
+    lo = torch.randn(2, 64, 5, 5, generator=g) * torch.rand(2, 1, 5, 5, generator=g).mul(12).sub(12).exp2()
+    lo[0, :32, 0, 0] = 0.0
+    q = Q.quant_lo_blocks(lo)
+    assert torch.count_nonzero(q[0, :32, 0, 0]) == 0
+    v, qv = lo.view(2, 2, 32, 5, 5), q.view(2, 2, 32, 5, 5)
+    sc = Q.block_scale(v.abs().amax(2, keepdim=True))
+    r = (v / sc).abs()
+    step = torch.where(r < 2, 0.125, torch.where(r < 4, 0.25, 0.5))
+    ok = ((qv - v).abs() <= 0.5 * step * sc * (1 + 1e-6)) | (r > 7.5)   # saturated elements aside
+    assert bool(ok.all())
+    assert bool(((qv / sc).abs() <= 7.5).all())
+
+
+def test_bf16f6_emulation_reduces_to_the_bf16_emulation_and_to_bf16_weights():
+    st = R.init_state(4, "reference")
+    x, legal = gen_boards(6, 200, 3)
+    x[1, 2] = torch.rand(19, 19, generator=torch.Generator().manual_seed(1))     # a varying third plane too
+    with torch.inference_mode():
+        # no layer corrected: exactly the plain bf16 contract
+        l0, v0 = Q.forward_bf16f6_emulated(st, x, lo_mask=0)
+        le, ve = R.forward_bf16_emulated(st, x, act_scale=Q.ACT_SCALE, exact_constant_plane=True)
+        assert torch.equal(l0, le) and torch.equal(v0, ve)
+        # exact low-order parts: the forward with bf16 weights and unrounded activations (the
+        # first layer's constant plane aside, which the kernels keep unrounded: both forms here)
+        lx, _ = Q.forward_bf16f6_emulated(st, x, exact_lo=True, exact_constant_plane=False)
+        stq = {k: (v.to(torch.bfloat16).float() if k.startswith("convs.") and k.endswith("weight") else v)
+               for k, v in st.items()}
+        # (the first layer's weights are rounded after the activation scale is folded into them)
+        stq["convs.0.weight"] = (st["convs.0.weight"] * Q.ACT_SCALE).to(torch.bfloat16).float() / Q.ACT_SCALE
+        lw, _ = R.forward(stq, x.to(torch.bfloat16).float())
+        assert float((lx - lw).norm() / lw.norm()) < 2e-5
+        # the fp6 correction sits between the two
+        l6, _ = Q.forward_bf16f6_emulated(st, x, exact_constant_plane=False)
+        e_plain = float((le - lw).norm() / lw.norm())
+        e_f6 = float((l6 - lw).norm() / lw.norm())
+        assert e_f6 < 0.25 * e_plain
+
+
+def test_cascade_rule_against_a_plain_python_loop():
+    g = torch.Generator().manual_seed(9)
+    logits = torch.randn(40, 361, generator=g) * torch.rand(40, 1, generator=g) + 3.0 * torch.randn(40, 1, generator=g)
+    free = torch.rand(40, 361, generator=g) < 0.6
+    logits[0] = 0.25                                   # flat: no spread, no second pass
+    free[1] = False; free[1, 17] = True                # one free square: nothing to decide
+    free[2] = False                                    # none
+    logits[3, 5] = logits[3, 200] = 50.0; free[3, 5] = free[3, 200] = True   # a tie at the top
+    for thr in (0.0, 0.03, 0.5, -1.0):
+        got = Q.cascade_second_pass(logits, free, thr).tolist()
+        for b in range(40):
+            z = sorted((float(logits[b, i]) for i in range(361) if bool(free[b, i])), reverse=True)
+            if len(z) < 2:
+                want = False
+            elif thr < 0:
+                want = True
+            else:
+                mean = sum(z) / len(z)
+                std = math.sqrt(sum((v - mean) ** 2 for v in z) / len(z))
+                want = (z[0] - z[1]) < thr * std
+            assert got[b] == want, (thr, b)
+    assert Q.cascade_second_pass(logits, free, 0.03)[3] and not Q.cascade_second_pass(logits, free, 0.03)[0]
