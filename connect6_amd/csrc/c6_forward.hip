@@ -17,26 +17,8 @@
 
 namespace c6 {
 
-// Optional phase timestamps for kernel tuning (never compiled into the shipped library).
-#ifdef C6_DUMP_POINT
-__device__ unsigned g_dump[48 * 1024];
-extern "C" int c6_debug_dump(unsigned *host_out) {
-  return (int)hipMemcpyFromSymbol(host_out, HIP_SYMBOL(g_dump), sizeof(unsigned) * 48 * 1024);
-}
-// copy the first 128 KiB of LDS (+ optionally one lane-private value per thread) of workgroup 0
-#define C6_DUMP(point, smem, val)                                                          \
-  do {                                                                                     \
-    if ((point) == C6_DUMP_POINT && blockIdx.x == 0 && trace_on) {                         \
-      __syncthreads();                                                                     \
-      for (int i_ = threadIdx.x; i_ < 32 * 1024; i_ += 256)                                \
-        g_dump[i_] = reinterpret_cast<const unsigned *>(smem)[i_];                         \
-      g_dump[32 * 1024 + threadIdx.x] = (val);                                             \
-      __syncthreads();                                                                     \
-    }                                                                                      \
-  } while (0)
-#else
-#define C6_DUMP(point, smem, val) do { } while (0)
-#endif
+// Optional phase timestamps for kernel tuning (connect6_amd/profiling.py builds a traced copy;
+// the shipped library contains none of this).
 #ifdef C6_TRACE
 __device__ long long g_trace[256 * 4 * 64];
 #define C6_MARK(idx)                                                                       \
@@ -59,12 +41,6 @@ template <class P> __device__ __forceinline__ void mma(const v4i &a, const v4i &
 template <> __device__ __forceinline__ void mma<PrecBF16>(const v4i &a, const v4i &b, f32x16 &c) {
   c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
                                               __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-}
-template <> __device__ __forceinline__ void mma<PrecBF16X2>(const v4i &a, const v4i &b, f32x16 &c) {
-  mma<PrecBF16>(a, b, c);
-}
-template <> __device__ __forceinline__ void mma<PrecBF16F8>(const v4i &a, const v4i &b, f32x16 &c) {
-  mma<PrecBF16>(a, b, c);
 }
 template <> __device__ __forceinline__ void mma<PrecBF16F6>(const v4i &a, const v4i &b, f32x16 &c) {
   mma<PrecBF16>(a, b, c);
@@ -110,7 +86,7 @@ struct DropConsts {
 };
 template <class P> __device__ __forceinline__ DropConsts drop_consts() {
   unsigned b0 = 0x0000BF80u, b1 = 0xBF800000u;
-  if constexpr (P::LO8) asm volatile("" : "+v"(b0), "+v"(b1));  // (only the modes that use them)
+  if constexpr (P::LO6) asm volatile("" : "+v"(b0), "+v"(b1));  // (only the mode that uses them)
   return DropConsts{__builtin_bit_cast(bf16x2, b0), __builtin_bit_cast(bf16x2, b1)};
 }
 __device__ __forceinline__ float dropped_lo(float a, int w, const DropConsts &k) {
@@ -131,41 +107,19 @@ template <class P> __device__ __forceinline__ int swz_of(int pos) {
 
 // four consecutive channels of one position, converted to the storage type
 template <class P> struct Packed4 {
-  v2i hi;  // 16-bit modes: 4 values; split mode: the leading bf16 parts
-  v2i lo;  // split mode only: what the first rounding dropped
+  v2i hi;  // 16-bit modes: 4 values
 };
 template <> struct Packed4<PrecF32> {
   f32x4 v;
 };
 
-template <class P> __device__ __forceinline__ Packed4<P> pack4(const float (&v)[4], const DropConsts &k) {
+template <class P> __device__ __forceinline__ Packed4<P> pack4(const float (&v)[4]) {
   Packed4<P> r;
   if constexpr (P::EB == 4) {
     r.v = f32x4{v[0], v[1], v[2], v[3]};
   } else {
     r.hi[0] = pack2<P>(v[0], v[1]);
     r.hi[1] = pack2<P>(v[2], v[3]);
-    if constexpr (P::SPLIT) {
-      // (unpack and subtract here: the dot2 form measured 1.7 % slower in this mode)
-      r.lo[0] = pack2<P>(v[0] - __builtin_bit_cast(float, r.hi[0] << 16),
-                         v[1] - __builtin_bit_cast(float, r.hi[0] & (int)0xffff0000));
-      r.lo[1] = pack2<P>(v[2] - __builtin_bit_cast(float, r.hi[1] << 16),
-                         v[3] - __builtin_bit_cast(float, r.hi[1] & (int)0xffff0000));
-    }
-    if constexpr (P::LO8 && !P::LO6) {  // dropped low-order parts as four e4m3 bytes of lo * 2^kLoScaleLog2
-      // v_cvt_scalef32_pk_fp8_f32 divides by its scale operand and turns overflow into NaN,
-      // so the inputs are clamped to what 448 * 2^-kLoScaleLog2 can represent.
-      constexpr float INV = 1.0f / (float)(1 << kLoScaleLog2), LIM = 448.0f * INV;
-      typedef short v2s __attribute__((ext_vector_type(2)));
-      const float l0 = __builtin_amdgcn_fmed3f(dropped_lo(v[0], r.hi[0], k), -LIM, LIM);
-      const float l1 = __builtin_amdgcn_fmed3f(dropped_hi(v[1], r.hi[0], k), -LIM, LIM);
-      const float l2 = __builtin_amdgcn_fmed3f(dropped_lo(v[2], r.hi[1], k), -LIM, LIM);
-      const float l3 = __builtin_amdgcn_fmed3f(dropped_hi(v[3], r.hi[1], k), -LIM, LIM);
-      v2s w = {0, 0};
-      w = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(w, l0, l1, INV, false);
-      w = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(w, l2, l3, INV, true);
-      r.lo[0] = __builtin_bit_cast(int, w);
-    }
   }
   return r;
 }
@@ -178,10 +132,6 @@ __device__ __forceinline__ void put4(unsigned char *smem, int pbase, int sw, int
     *reinterpret_cast<f32x4 *>(smem + pbase + (o ^ sw)) = r.v;
   } else {
     *reinterpret_cast<v2i *>(smem + pbase + (o ^ sw)) = r.hi;
-    if constexpr (P::SPLIT)
-      *reinterpret_cast<v2i *>(smem + pbase + ((o + Geo<P>::PLANE) ^ sw)) = r.lo;
-    if constexpr (P::LO8 && !P::LO6)  // one byte per channel: channel index = o / 2
-      *reinterpret_cast<int *>(smem + pbase + Geo<P>::LO_OFF + (o >> 1)) = r.lo[0];
   }
 }
 
@@ -278,9 +228,6 @@ template <int B, int E, class F> __device__ __forceinline__ void static_for(F &&
   }
 }
 
-#ifndef C6_X_LO_NUM
-#define C6_X_LO_NUM 8
-#endif
 constexpr int kAhead = 2;  // k-steps between the LDS read of an activation fragment and its MFMAs
 
 // Issue order inside one k-step: memory instructions are dealt out one at a time between
@@ -407,14 +354,11 @@ __device__ __forceinline__ void conv3_pass(const unsigned char *smem, const WFra
   };
   set_row(0);
   static_assert(U % (kAhead + 1) == 0 && kAhead <= KC, "fragment queue must line up across kernel rows");
-  v4i bq[kAhead + 1][3], lq[kAhead + 1][3];
+  v4i bq[kAhead + 1][3];
 #pragma unroll
   for (int a = 0; a < kAhead; ++a)
 #pragma unroll
-    for (int j = 0; j < 3; ++j) {
-      bq[a][j] = frag_at(j, 0, a * 32);
-      if constexpr (P::SPLIT) lq[a][j] = frag_at(j, 0, a * 32 + G::PLANE);
-    }
+    for (int j = 0; j < 3; ++j) bq[a][j] = frag_at(j, 0, a * 32);
 
 #pragma unroll 1
   for (int ky = 0; ky < 3; ++ky) {
@@ -428,55 +372,38 @@ __device__ __forceinline__ void conv3_pass(const unsigned char *smem, const WFra
       const int un = (u + kAhead) % U;
       const int kxn = un / KC, on = (un % KC) * 32;
 #pragma unroll
-      for (int j = 0; j < 3; ++j) {
-        bq[(u + kAhead) % QN][j] = frag_at(j, kxn, on);
-        if constexpr (P::SPLIT) lq[(u + kAhead) % QN][j] = frag_at(j, kxn, on + G::PLANE);
-      }
+      for (int j = 0; j < 3; ++j) bq[(u + kAhead) % QN][j] = frag_at(j, kxn, on);
 #pragma unroll
       for (int t = 0; t < NT; ++t)
 #pragma unroll
         for (int j = 0; j < 3; ++j) mma<P>(ring[u % D][t], bq[u % QN][j], acc[t][j]);
-      if constexpr (P::SPLIT) {
-#pragma unroll
-        for (int t = 0; t < NT; ++t)
-#pragma unroll
-          for (int j = 0; j < 3; ++j) mma<P>(ring[u % D][t], lq[u % QN][j], acc[t][j]);
-      }
       // weights of k-step u+D (the tail over-reads into the next layer)
 #pragma unroll
       for (int t = 0; t < NT; ++t) ring[u % D][t] = wn[u * NT + t];
-      interleave_step<NT * 3 * (P::SPLIT ? 2 : 1) * (P::EB == 4 ? 4 : 1), 3 * (P::SPLIT ? 2 : 1), NT>();
+      interleave_step<NT * 3 * (P::EB == 4 ? 4 : 1), 3, NT>();
       __builtin_amdgcn_sched_barrier(0);
     }
   }
 }
 
-// Second pass of the bf16 + fp8 / fp6 modes over a 3x3 layer: acc += Wlo * LO, both e4m3 (or
-// both e2m3), K = 64 per MFMA.  Lane half h of chunk c contracts half-chunk g = 2c + h =
-// (tap, 32-channel block); in the fp6 mode the block's scale byte rides in dword 6 of the
-// 32 bytes the lane reads.
+// Second pass of the bf16 + fp6 mode over a 3x3 layer: acc += Wlo * LO, both e2m3, K = 64 per
+// MFMA.  Lane half h of chunk c contracts half-chunk g = 2c + h = (tap, 32-channel block); the
+// block's scale byte rides in dword 6 of the 32 bytes the lane reads.
 //
-// Its weight ring: a lane's operand is 32 bytes (fp8) or 24 (fp6), piece 0 = 16 bytes and
-// piece 1 = 16 or 8.  (Filling the ring before the layer's main pass was measured slower: the
-// extra loads and registers cost the main pass more than the second pass gains.)
+// Its weight ring: a lane's operand is 24 bytes, piece 0 = 16 bytes and piece 1 = 8.  (Filling
+// the ring before the layer's main pass was measured slower: the extra loads and registers cost
+// the main pass more than the second pass gains.)
 template <class P>
 __device__ __forceinline__ void lo_load_pieces(const WFrags &src, v4i &p0, v4i &p1) {
   p0 = src[0];
-  if constexpr (P::LO6) {
-    const v2i q = src.dense8(1);
-    p1 = v4i{q[0], q[1], 0, 0};
-  } else {
-    p1 = src[1];
-  }
+  const v2i q = src.dense8(1);
+  p1 = v4i{q[0], q[1], 0, 0};
 }
 template <class P, int L> struct LoRing {
   static constexpr int NT = kCoutArr[L] / 32;
   static constexpr int NC = Geo<P>::lo_chunks(L);
-#ifndef C6_LO_DEEP
-#define C6_LO_DEEP 3
-#endif
   // ring depth in 64-wide chunks: the weights of a chunk are asked for D chunks before its MFMAs
-  static constexpr int D = !P::LO8 ? 1 : (P::PIPE && NC >= 9 ? C6_LO_DEEP : (NC < kLoRing ? NC : kLoRing));
+  static constexpr int D = P::LO6 ? kLoRing : 1;
   __device__ __forceinline__ static WFrags base(const unsigned char *packed, int lane) {
     return packed_frags<P>(packed, lane, Geo<P>::lo_frag_offset(L));
   }
@@ -496,13 +423,13 @@ __device__ __forceinline__ void lo_preload(v4i (&f0)[D][NT], v4i (&f1)[D][NT],
 // A runtime loop over groups of D chunks (D = ring depth) keeps the compiler from hoisting
 // every fragment load of the layer to the front.
 //   INIT: the accumulators are undefined on entry; the first chunk's MFMAs start from `bias`
-//   BYTE_BASE: `ci` holds byte addresses (position record + 8 * lane half, what the epilogue
-//   stores through) instead of position indices: no address registers of the pass's own
-template <class P, int L, bool INIT, bool BYTE_BASE, int D, int NT>
+//   wb[j]: byte address of the lane's position record + 8 * lane half (what the epilogue stores
+//   through): the pass has no address registers of its own
+template <class P, int L, bool INIT, int D, int NT>
 __device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
                                               const unsigned char *packed, int scale_w,
                                               v4i (&ring0)[D][NT], v4i (&ring1)[D][NT],
-                                              const int (&ci)[3], int h, int lane,
+                                              const int (&wb)[3], int h, int lane,
                                               f32x16 (&acc)[NT][3], const f32x16 (&bias)[NT]) {
   using G = Geo<P>;
   static_assert(D == LoRing<P, L>::D && NT == kCoutArr[L] / 32, "ring shape");
@@ -513,13 +440,8 @@ __device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
   // scale_w: E8M0 exponent undoing the weight copy's 2^sw.  (It arrives as an argument, read once
   // per board: a load here would be the newest of ~36 loads in flight, and waiting for it before the
   // first MFMA would drain them all.)
-  const int scale_x = 127 - kLoScaleLog2;  // ... and the activations' 2^kLoScaleLog2 (fp8 mode)
-  (void)scale_x;
 
-  int pbase[3];
-#pragma unroll
-  for (int j = 0; j < 3; ++j) pbase[j] = BYTE_BASE ? ci[j] : ci[j] * G::PIXB + G::LO_OFF;
-  // Byte offset of a half-chunk relative to pbase[].  Half-chunk g = 2 c + (lane half) of chunk
+  // Byte offset of a half-chunk relative to wb[].  Half-chunk g = 2 c + (lane half) of chunk
   // c = 3 grp + dd is g = 6 grp + r with r = 2 dd + half: with `r` a constant, the tap and the
   // channel block of g need no division by the tile count, and for 64 input channels (6
   // half-chunks = 3 taps = one kernel row) no division at all.  The group number may be a
@@ -546,7 +468,7 @@ __device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
       ky = 2 * grp + r / 3;
       kx = r % 3;
     }
-    return ((ky - 1) * kPitch + (kx - 1)) * G::PIXB + cb * 32 + (BYTE_BASE ? G::LO_OFF : 0);
+    return ((ky - 1) * kPitch + (kx - 1)) * G::PIXB + cb * 32 + G::LO_OFF;
   };
   // chunk 3 grp + dd; STATIC: grp is a constant after unrolling, and the chunk may lie beyond the
   // last one (harmless re-reads of the last) or hold the padding half-chunk (which re-reads the
@@ -559,40 +481,26 @@ __device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
       o1 = off_g(g1 / 6, g1 % 6);
     };
     int o0, o1;
-    if constexpr (!BYTE_BASE) {
-      // (the layer-by-layer kernels: one formula on the lane's own half-chunk number; the
-      // scalar form below costs them registers)
-      int c = D * grp + dd;
-      c = c < NC ? c : NC - 1;
-      int g = 2 * c + hh;
-      g = g < HC ? g : HC - 1;
-      const int tap = g / PER32, cb = g - tap * PER32;
-      const int ky = tap / 3, kx = tap - 3 * ky;
-      o0 = o1 = ((ky - 1) * kPitch + (kx - 1)) * G::PIXB + cb * 32;
-    } else if constexpr (decltype(is_static)::value) {
+    if constexpr (decltype(is_static)::value) {
       of_chunk(D * grp + dd, o0, o1);
     } else {
       // (run-time group: never the last chunk nor beyond it, see the loop bounds below)
       o0 = off_g(grp, 2 * dd);
       o1 = off_g(grp, 2 * dd + 1);
     }
-    const int off = hh ? o1 - (BYTE_BASE ? 8 : 0) : o0;
+    const int off = hh ? o1 - 8 : o0;
 #pragma unroll
     for (int j = 0; j < 3; ++j) {
-      b[j][0] = *reinterpret_cast<const v4i *>(smem + pbase[j] + off);
-      if constexpr (P::LO6) {
-        // The last two data dwords with an 8-byte read, straight into the operand's registers 4
-        // and 5, and the scale on its own (volatile: the compiler would merge the two into one
-        // 12-byte read again, whose three registers cannot be part of the six-register operand,
-        // and copy two of them; a 16-byte read would leave a dead register that the compiler
-        // reuses at once, waiting for the read to land first).
-        const v2i q = *reinterpret_cast<const v2i *>(smem + pbase[j] + off + 16);
-        typedef const volatile __attribute__((address_space(3))) int *LdsVolatileInt;
-        const int sc = *(LdsVolatileInt)(smem + pbase[j] + off + 24);
-        b[j][1] = v4i{q[0], q[1], sc, sc};
-      } else {
-        b[j][1] = *reinterpret_cast<const v4i *>(smem + pbase[j] + off + 16);
-      }
+      b[j][0] = *reinterpret_cast<const v4i *>(smem + wb[j] + off);
+      // The last two data dwords with an 8-byte read, straight into the operand's registers 4
+      // and 5, and the scale on its own (volatile: the compiler would merge the two into one
+      // 12-byte read again, whose three registers cannot be part of the six-register operand,
+      // and copy two of them; a 16-byte read would leave a dead register that the compiler
+      // reuses at once, waiting for the read to land first).
+      const v2i q = *reinterpret_cast<const v2i *>(smem + wb[j] + off + 16);
+      typedef const volatile __attribute__((address_space(3))) int *LdsVolatileInt;
+      const int sc = *(LdsVolatileInt)(smem + wb[j] + off + 24);
+      b[j][1] = v4i{q[0], q[1], sc, sc};
     }
   };
   // activation blocks are fetched kAhead chunks ahead, like the main pass's fragments
@@ -605,9 +513,7 @@ __device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
   auto chunk = [&](int grp, int d, auto first, auto is_static) __attribute__((always_inline)) {
     const WFrags wn = wl + (grp + 1) * (D * NT * 2);
     v4i(&bcur)[3][2] = bq[d % (kAhead + 1)];
-#ifndef C6_X_NOLOA
     fetch(grp + (d + kAhead) / D, (d + kAhead) % D, is_static, bq[(d + kAhead) % (kAhead + 1)]);
-#endif
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       const v8i a = __builtin_shufflevector(ring0[d][t], ring1[d][t], 0, 1, 2, 3, 4, 5, 6, 7);
@@ -620,28 +526,22 @@ __device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
         } else {
           c = acc[t][j];
         }
-        if constexpr (P::LO6) {
-          acc[t][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 2, 2, 0, scale_w, 0, b[6]);
-        } else {
-          acc[t][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, scale_w, 0, scale_x);
-        }
+        acc[t][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 2, 2, 0, scale_w, 0, b[6]);
       }
     }
     // weights of chunk c0 + d + D (the tail over-reads the next layer's copy or the zero padding)
-#ifndef C6_X_NOLOW
 #pragma unroll
     for (int t = 0; t < NT; ++t) lo_load_pieces<P>(wn + (d * NT + t) * 2, ring0[d][t], ring1[d][t]);
-#endif
     interleave_step<NT * 3, 2 * 3, 2 * NT>();
     __builtin_amdgcn_sched_barrier(0);
   };
   // Whole groups of D chunks in a runtime loop with a single basic block (a branch inside the
   // body makes the compiler wait for every LDS read in flight at each group boundary), then the
-  // chunks that are left, unrolled.  With the scalar offsets (BYTE_BASE) the loop only takes the
-  // groups whose reads ahead stay in front of the last chunk, so that its body needs neither of
-  // the two special cases (a select per read costs more than the longer unrolled tail).
+  // chunks that are left, unrolled.  The loop only takes the groups whose reads ahead stay in
+  // front of the last chunk, so that its body needs neither of the two special cases (a select
+  // per read costs more than the longer unrolled tail).
   constexpr int LIM = NC - 2 - (D - 1) - kAhead;  // last chunk such a group may start at
-  constexpr int GROUPS = BYTE_BASE ? (LIM >= 0 ? LIM / D + 1 : 0) : NC / D;
+  constexpr int GROUPS = LIM >= 0 ? LIM / D + 1 : 0;
   constexpr int FIRST = INIT ? 1 : 0;
   static_assert(NC >= D, "at least one whole group");
   if constexpr (INIT) {  // (the first group apart: its first chunk initialises the accumulators)
@@ -661,12 +561,11 @@ __device__ __forceinline__ void conv3_lo_pass(const unsigned char *smem,
 
 // SiLU of the four accumulators (tile t, pixel tile j, quad q): bias was added at init
 template <class P, int NT>
-__device__ __forceinline__ Packed4<P> silu_quad(const f32x16 (&acc)[NT][3], int t, int j, int q,
-                                                 const DropConsts &k) {
+__device__ __forceinline__ Packed4<P> silu_quad(const f32x16 (&acc)[NT][3], int t, int j, int q) {
   float v[4];
 #pragma unroll
   for (int e = 0; e < 4; ++e) v[e] = silu<P>(acc[t][j][4 * q + e]);
-  return pack4<P>(v, k);
+  return pack4<P>(v);
 }
 
 // SiLU + store of one pixel tile's accumulators (all cout tiles).  Lanes beyond pixel
@@ -681,12 +580,11 @@ __device__ __forceinline__ void store_tile(unsigned char *smem, int pos_in, int 
   asm volatile("" : "+v"(pos));
   const int pbase = pos * G::PIXB;
   const int sw = swz_of<P>(pos);
-  const DropConsts k = drop_consts<P>();
 #pragma unroll
   for (int t = 0; t < NT; ++t)
 #pragma unroll
     for (int q = 0; q < 4; ++q)
-      put4<P>(smem, pbase, sw, (32 * t + 8 * q + 4 * h) * G::EB, silu_quad<P, NT>(acc, t, j, q, k));
+      put4<P>(smem, pbase, sw, (32 * t + 8 * q + 4 * h) * G::EB, silu_quad<P, NT>(acc, t, j, q));
 }
 
 // fp6 mode: 32 low-order values of one position -> 24 bytes of e2m3 + the block's E8M0 scale.
@@ -765,8 +663,7 @@ __device__ __forceinline__ void load_bias_tiles_lds(f32x16 (&bt)[N], const unsig
 }
 
 // barrier; every wave writes its share of the layer's output over the layer's input; barrier
-// (WITH_LO: the next layer runs a low-order pass, so its input needs the low-order part)
-template <class P, int NT, bool WITH_LO, class Pre>
+template <class P, int NT, class Pre>
 __device__ __forceinline__ void finish_layer(unsigned char *smem, const int (&ci)[3], int h,
                                              const f32x16 (&acc)[NT][3], Pre before_store) {
   __syncthreads();  // every wave has finished reading the layer's input
@@ -776,31 +673,23 @@ __device__ __forceinline__ void finish_layer(unsigned char *smem, const int (&ci
   __syncthreads();
 }
 
-// one 3x3 layer that is not the last
+// one 3x3 layer that is not the last (layer-by-layer kernel)
 template <class P, int L>
 __device__ __forceinline__ void mid_layer(
     unsigned char *smem, const unsigned char *packed, const float *tail,
     v4i (&ring)[kRing][kCoutArr[L] / 32], v4i (&next)[kRing][kCoutArr[L + 1] / 32],
-    const int (&ci)[3], int h, int lane, int wave, bool trace_on, const int (&lo_scale_w)[8]) {
+    const int (&ci)[3], int h, int lane, int wave, bool trace_on) {
   constexpr int CIN = kCinArr[L], COUT = kCoutArr[L], NT = COUT / 32;
   f32x16 acc[NT][3];
   init_acc(acc, tail + bias_offset(L), h);
-  v4i lor0[LoRing<P, L>::D][LoRing<P, L>::NT], lor1[LoRing<P, L>::D][LoRing<P, L>::NT];
   conv3_pass<P, CIN, COUT>(smem, layer_weights<P, L>(packed, lane), ring, ci, h, acc);
   C6_MARK(30 + L);
-  if constexpr (P::LO8 && L >= P::LO_FIRST) {
-    lo_preload<P, L>(lor0, lor1, packed, lane);
-    {
-      f32x16 nobias[NT];
-      conv3_lo_pass<P, L, false, false>(smem, packed, lo_scale_w[L], lor0, lor1, ci, h, lane, acc, nobias);
-    }
-  }
   // With equal channel counts the main pass's over-read has already left the next layer's first
   // kRing k-steps in the ring (same fragment order, contiguous in memory): `next` is `ring`.
   if constexpr (kCoutArr[L + 1] != kCoutArr[L])
     preload_ring<kRing, kCoutArr[L + 1] / 32>(next, layer_weights<P, L + 1>(packed, lane));
   C6_MARK(4 + 2 * L);
-  finish_layer<P, NT, (L + 1 >= P::LO_FIRST)>(smem, ci, h, acc, [] {});
+  finish_layer<P, NT>(smem, ci, h, acc, [] {});
   C6_MARK(5 + 2 * L);
   (void)wave;
   (void)trace_on;
@@ -924,15 +813,6 @@ __device__ __forceinline__ void epi_atom(unsigned char *smem, const int (&wb)[3]
                                          EpiCarry &c, const DropConsts &k) {
   using G = Geo<P>;
   const int kind = code >> 8, idx = code & 255;
-#ifdef C6_EXP_SKIP  // (tuning builds: leave out kinds of hidden atoms; results are wrong)
-  if constexpr (UNDER_MFMA) {
-    if ((C6_EXP_SKIP & 1) && kind == kAtW) return;
-    if ((C6_EXP_SKIP & 2) && kind >= kAtF1) return;
-    if ((C6_EXP_SKIP & 4) && (kind == kAtD || kind == kAtX)) return;
-    if ((C6_EXP_SKIP & 8) && kind == kAtF3) return;
-    if ((C6_EXP_SKIP & 16) && kind <= kAtM) return;
-  }
-#endif
   auto tile_of = [](int n) __attribute__((always_inline)) { return n / R::CNT; };
   auto reg_of = [](int n) __attribute__((always_inline)) { return R::I0 + n % R::CNT; };
   if (kind == kAtE) {
@@ -1112,7 +992,7 @@ __device__ __forceinline__ void conv3_seg(const unsigned char *smem, const WFrag
     constexpr int u = g / (NTS * 3), ti = (g / 3) % NTS, t = T0 + ti, j = g % 3;
     constexpr int f = F0 + u * NTS + ti;
     // (a layer with one input tile runs its low-order pass first, and that one starts from the bias)
-    constexpr bool kLoFirst = P::LO8 && ((P::LO_MASK >> L) & 1) && NTP == 1;
+    constexpr bool kLoFirst = P::LO6 && ((P::LO_MASK >> L) & 1) && NTP == 1;
     if constexpr (PH == 0 && u == 0 && !kLoFirst) {
       f32x16 c0 = bias[t];
       mma<P>(ring[f % RN], bq[(KS0 + u) % QN][j], c0);
@@ -1162,10 +1042,8 @@ __device__ __forceinline__ void pipe_layer(
   f32x16 bias[NT];
   v4i bq[kAhead + 1][3];
   using Whole = EpiRange<0, 16>;
-  // (the low-order weight ring is filled in front of the barrier that precedes its pass; filling
-  // it a whole phase earlier costs that phase what the pass gains)
-  constexpr bool kLoPass = P::LO8 && ((P::LO_MASK >> L) & 1);
-  constexpr bool kLoNext = P::LO8 && L + 1 < kLayers && ((P::LO_MASK >> (L + 1)) & 1);  // this layer's output needs its low-order part
+  constexpr bool kLoPass = P::LO6 && ((P::LO_MASK >> L) & 1);
+  constexpr bool kLoNext = P::LO6 && L + 1 < kLayers && ((P::LO_MASK >> (L + 1)) & 1);  // this layer's output needs its low-order part
   v4i lor0[LoRing<P, L>::D][LoRing<P, L>::NT], lor1[LoRing<P, L>::D][LoRing<P, L>::NT];
   __syncthreads();  // every wave has finished layer L-1 (its reads, and tile 0 if it stored it there)
   if constexpr (NTP == 1) {
@@ -1183,34 +1061,23 @@ __device__ __forceinline__ void pipe_layer(
     load_bias_tiles_lds(bias, smem, tail_lds, bias_offset(L), h);
   }
   C6_MARK(L == 1 ? 3 : 3 + 2 * L);
-  C6_DUMP(10 + L, smem, __builtin_bit_cast(unsigned, prev[0][0][0]));
   const WFrags wl = layer_weights<P, L>(packed, lane);
   // phases 0 .. NTP-2 carry tiles 1 .. NTP-1 of layer L-1
   static_for<0, NTP - 1>([&](auto pc) __attribute__((always_inline)) {
     constexpr int p = decltype(pc)::value;
     using Plan = EpiPlan<P, Whole, kLoPass, true, kPhaseSteps * NT * 3 - 8>;
-    // The last of these phases also asks for the low-order pass's first weights, one ring slot
-    // every few MFMAs over its second half: in one burst in front of the barrier the pass starts
-    // by waiting a round trip to L2, and in one burst earlier the loads hold up the phase's own
-    // fragments (the vector memory counter is served in order).
-    constexpr int SLOTS = kPhaseSteps * NT * 3, NLOAD = LoRing<P, L>::D * NT;
-    constexpr int LO_G0 = SLOTS * (C6_X_LO_NUM < 8 ? C6_X_LO_NUM : 0) / 8, LO_STRIDE = (SLOTS - 12 - LO_G0) / NLOAD;
-    static_assert(LO_STRIDE >= 1, "room for the low-order ring loads");
-    const WFrags lo_wl = LoRing<P, L>::base(packed, lane);
     conv3_seg<P, L, kSegFull, p>(smem, wl, ring, bq, rb, acc, bias, [&](int g) __attribute__((always_inline)) {
       Plan::template run<NTP>(smem, wb, h4, prev, p + 1, (RIN + p + 1) % 3, g, carry, k);
-      if constexpr (kLoPass && p == NTP - 2 && C6_X_LO_NUM < 8) {
-        const int i = (g - LO_G0) / LO_STRIDE;
-        if (g >= LO_G0 && (g - LO_G0) % LO_STRIDE == 0 && i < NLOAD)
-          lo_load_pieces<P>(lo_wl + i * 2, lor0[i / NT][i % NT], lor1[i / NT][i % NT]);
-      }
     });
-    if constexpr (kLoPass && p == NTP - 2 && C6_X_LO_NUM >= 8) lo_preload<P, L>(lor0, lor1, packed, lane);
+    // (The low-order weight ring is filled in one burst in front of the barrier that precedes its
+    // pass.  Dealt out over this phase's MFMA slots instead, the phase gets 4 % shorter and the
+    // kernel no faster, for two or three spilled registers.)
+    if constexpr (kLoPass && p == NTP - 2) lo_preload<P, L>(lor0, lor1, packed, lane);
     __syncthreads();
   });
   C6_MARK(30 + L);
   if constexpr (kLoPass) {
-    conv3_lo_pass<P, L, NTP == 1, true>(smem, packed, lo_scale_w[L], lor0, lor1, wb, h, lane, acc, bias);
+    conv3_lo_pass<P, L, NTP == 1>(smem, packed, lo_scale_w[L], lor0, lor1, wb, h, lane, acc, bias);
     // before part B overwrites fp6 block 0, every wave must have read it
     if constexpr (NT > 1 && !kLast) __syncthreads();
   }
@@ -1229,7 +1096,6 @@ __device__ __forceinline__ void pipe_layer(
     });
   }
   C6_MARK(4 + 2 * L);
-  C6_DUMP(20 + L, smem, __builtin_bit_cast(unsigned, acc[0][0][0]));
   (void)wave;
   (void)trace_on;
 }
@@ -1402,14 +1268,12 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
     // block-scale exponents of the low-order weight copies (E8M0: 127 - log2 of the copy's scale),
     // fetched here, long before any second pass needs them
     int lo_scale_w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    if constexpr (P::LO8) {
+    if constexpr (P::LO6) {
 #pragma unroll
       for (int l = 1; l < 8; ++l) lo_scale_w[l] = 127 - reinterpret_cast<const int *>(tail)[G::TAIL_SW + l];
     }
 
-#if defined(C6_DUMP_POINT)
-    const bool trace_on = (it == it_first + 1);  // second board of this workgroup
-#elif defined(C6_TRACE)
+#if defined(C6_TRACE)
     const bool trace_on = (it == it_first + 2);  // third board of this workgroup
 #else
     const bool trace_on = false;
@@ -1811,14 +1675,6 @@ __global__ __launch_bounds__(256) void fused_forward_kernel(const FwdParams prm)
     asm volatile("" : "+v"(tidv));
     const unsigned char *packed = packed_of(b);
     const float *tail = reinterpret_cast<const float *>(packed + G::TAIL_OFF);
-    // block-scale exponents of the low-order weight copies (E8M0: 127 - log2 of the copy's scale),
-    // fetched here, long before any second pass needs them
-    int lo_scale_w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    if constexpr (P::LO8) {
-#pragma unroll
-      for (int l = 1; l < 8; ++l) lo_scale_w[l] = 127 - reinterpret_cast<const int *>(tail)[G::TAIL_SW + l];
-    }
-
 #ifdef C6_TRACE
     const bool trace_on = (b == b_first + 2);  // third board of this workgroup
 #else
@@ -1869,7 +1725,7 @@ __global__ __launch_bounds__(256) void fused_forward_kernel(const FwdParams prm)
       conv1_pass<P>(smem, layer_weights<P, 0>(packed, lane), r1, l1base, acc);
       preload_ring<kRing, 1>(r2, layer_weights<P, 1>(packed, lane));
       C6_MARK(2);
-      finish_layer<P, 1, (1 >= P::LO_FIRST)>(smem, ci, h, acc, [&] {
+      finish_layer<P, 1>(smem, ci, h, acc, [&] {
         // the copies overlapped the activation tile: restore its zero padding
         for (int i = tidv; i < 60 * (G::PIXB / 16); i += THREADS) {
           const int k = i / (G::PIXB / 16), w16 = i - k * (G::PIXB / 16);
@@ -1881,12 +1737,12 @@ __global__ __launch_bounds__(256) void fused_forward_kernel(const FwdParams prm)
       });
     }
     C6_MARK(3);
-    mid_layer<P, 1>(smem, packed, tail, r2, r345, ci, h, lane, wave, trace_on, lo_scale_w);
-    mid_layer<P, 2>(smem, packed, tail, r345, r345, ci, h, lane, wave, trace_on, lo_scale_w);
-    mid_layer<P, 3>(smem, packed, tail, r345, r345, ci, h, lane, wave, trace_on, lo_scale_w);
-    mid_layer<P, 4>(smem, packed, tail, r345, r678, ci, h, lane, wave, trace_on, lo_scale_w);
-    mid_layer<P, 5>(smem, packed, tail, r678, r678, ci, h, lane, wave, trace_on, lo_scale_w);
-    mid_layer<P, 6>(smem, packed, tail, r678, r678, ci, h, lane, wave, trace_on, lo_scale_w);
+    mid_layer<P, 1>(smem, packed, tail, r2, r345, ci, h, lane, wave, trace_on);
+    mid_layer<P, 2>(smem, packed, tail, r345, r345, ci, h, lane, wave, trace_on);
+    mid_layer<P, 3>(smem, packed, tail, r345, r345, ci, h, lane, wave, trace_on);
+    mid_layer<P, 4>(smem, packed, tail, r345, r678, ci, h, lane, wave, trace_on);
+    mid_layer<P, 5>(smem, packed, tail, r678, r678, ci, h, lane, wave, trace_on);
+    mid_layer<P, 6>(smem, packed, tail, r678, r678, ci, h, lane, wave, trace_on);
 
     // ---- layer 8 + both 1x1 heads straight from the fp32 accumulators ----
     {
@@ -1897,14 +1753,8 @@ __global__ __launch_bounds__(256) void fused_forward_kernel(const FwdParams prm)
       const float *pwl = polw + 4 * h;  // per-lane base: channel 32t + 8q + 4h + e
       asm volatile("" : "+v"(pwl));
       const GlobalF32 pwg = (GlobalF32)pwl;
-      v4i lor0[LoRing<P, 7>::D][LoRing<P, 7>::NT], lor1[LoRing<P, 7>::D][LoRing<P, 7>::NT];
       conv3_pass<P, 96, 96>(smem, layer_weights<P, 7>(packed, lane), r678, ci, h, acc);
       C6_MARK(37);
-      if constexpr (P::LO8) lo_preload<P, 7>(lor0, lor1, packed, lane);
-      if constexpr (P::LO8) {
-        f32x16 nobias[3];
-        conv3_lo_pass<P, 7, false, false>(smem, packed, lo_scale_w[7], lor0, lor1, ci, h, lane, acc, nobias);
-      }
       if (bn < b_end) preload_ring<L1Pipe<P>::D, 1>(r1, layer_weights<P, 0>(packed_of(bn), lane));
       C6_MARK(18);
       float pol[3] = {0.0f, 0.0f, 0.0f};
@@ -2041,7 +1891,7 @@ template <class P> __global__ void pack_kernel(const PackParams prm) {
         }
         return;
       }
-      if constexpr (P::LO8) {
+      if constexpr (P::LO6) {
         int ll = 1;
         while (ll < 8 && frag >= G::lo_frag_offset(ll + 1)) ++ll;
         if (frag >= G::HI_FRAGS && ll < 8) {
@@ -2053,31 +1903,19 @@ template <class P> __global__ void pack_kernel(const PackParams prm) {
             const int tap = g / per32, cb = g % per32, co = 32 * t + m;
             const float *w = prm.conv_w[ll];
             const float sc = exp2f((float)reinterpret_cast<const int *>(prm.packed + G::TAIL_OFF)[G::TAIL_SW + ll]);
-            if constexpr (P::LO6) {  // the lane's 32 K slots as e2m3: 24 bytes = piece 0 + half of piece 1
-              f32x16v even, odd;
+            // the lane's 32 K slots as e2m3 (the copy approximates the bf16 weights the main pass
+            // uses): 24 bytes = piece 0 + piece 1
+            f32x16v even, odd;
 #pragma unroll
-              for (int i = 0; i < 16; ++i) {
-                even[i] = (float)(__bf16)w[(co * cin + lo6_channel(cb, 2 * i)) * 9 + tap] * sc;
-                odd[i] = (float)(__bf16)w[(co * cin + lo6_channel(cb, 2 * i + 1)) * 9 + tap] * sc;
-              }
-              const u32x6 r = to_fp6_block(even, odd, 1.0f);
-              if (piece == 0) {
-                o = v4i{(int)r[0], (int)r[1], (int)r[2], (int)r[3]};
-              } else {
-                o = v4i{(int)r[4], (int)r[5], 0, 0};
-              }
-            } else
-#pragma unroll
-            for (int d = 0; d < 4; ++d) {
-              float v[4];
-#pragma unroll
-              for (int e = 0; e < 4; ++e) {
-                const int ch = cb * 32 + piece * 16 + d * 4 + e;
-                // the copy approximates the bf16 weights the main pass uses
-                v[e] = __builtin_amdgcn_fmed3f((float)(__bf16)w[(co * cin + ch) * 9 + tap] * sc, -448.0f, 448.0f);
-              }
-              int q = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], 0, false);
-              o[d] = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], q, true);
+            for (int i = 0; i < 16; ++i) {
+              even[i] = (float)(__bf16)w[(co * cin + lo6_channel(cb, 2 * i)) * 9 + tap] * sc;
+              odd[i] = (float)(__bf16)w[(co * cin + lo6_channel(cb, 2 * i + 1)) * 9 + tap] * sc;
+            }
+            const u32x6 r = to_fp6_block(even, odd, 1.0f);
+            if (piece == 0) {
+              o = v4i{(int)r[0], (int)r[1], (int)r[2], (int)r[3]};
+            } else {
+              o = v4i{(int)r[4], (int)r[5], 0, 0};
             }
           }
         }
@@ -2179,7 +2017,7 @@ template <class P> __global__ __launch_bounds__(256) void lo_scale_kernel(const 
   }
   if (threadIdx.x == 0) {
     int e = 0;
-    constexpr float kLargest = P::LO6 ? 7.5f : 448.0f;  // of e2m3 / e4m3
+    constexpr float kLargest = 7.5f;  // of e2m3
     if (red[0] > 0.0f && red[0] < INFINITY) e = (int)floorf(log2f(kLargest / red[0]));
     sw[l] = e < -20 ? -20 : (e > 20 ? 20 : e);
   }
@@ -2193,7 +2031,7 @@ template <class P> static int launch_pack(const PackParams &pp, hipStream_t st) 
   const long long total = (long long)G::TOTAL_FRAGS * 64 + G::TAIL_FLOATS;
   const int threads = 256;
   const int blocks = (int)((total + threads - 1) / threads);
-  if constexpr (P::LO8) hipLaunchKernelGGL(lo_scale_kernel<P>, dim3(8), dim3(256), 0, st, pp);
+  if constexpr (P::LO6) hipLaunchKernelGGL(lo_scale_kernel<P>, dim3(8), dim3(256), 0, st, pp);
   hipLaunchKernelGGL(pack_kernel<P>, dim3(blocks), dim3(threads), 0, st, pp);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
@@ -2257,8 +2095,6 @@ int dispatch_pack(int prec, const PackParams &pp, hipStream_t st) {
     case C6_PREC_F32: return launch_pack<PrecF32>(pp, st);
     case C6_PREC_BF16: return launch_pack<PrecBF16>(pp, st);
     case C6_PREC_F16: return launch_pack<PrecF16>(pp, st);
-    case C6_PREC_BF16X2: return launch_pack<PrecBF16X2>(pp, st);
-    case C6_PREC_BF16F8: return launch_pack<PrecBF16F8>(pp, st);
     case C6_PREC_BF16F6: return launch_pack<PrecBF16F6>(pp, st);
   }
   set_error("unknown precision mode %d", prec);
@@ -2266,23 +2102,14 @@ int dispatch_pack(int prec, const PackParams &pp, hipStream_t st) {
 }
 
 int dispatch_forward(int prec, const FwdParams &fp, hipStream_t st) {
-#ifdef C6_ONLY_BF16F6  // (tuning builds: compile few arithmetic modes only)
-  if (prec == C6_PREC_BF16F6) return launch_forward<PrecBF16F6>(fp, st);
-  if (prec == C6_PREC_BF16) return launch_forward<PrecBF16>(fp, st);
-  if (prec == C6_PREC_F32) return launch_forward<PrecF32>(fp, st);
-  return C6_EINVAL;
-#else
   switch (prec) {
     case C6_PREC_F32: return launch_forward<PrecF32>(fp, st);
     case C6_PREC_BF16: return launch_forward<PrecBF16>(fp, st);
     case C6_PREC_F16: return launch_forward<PrecF16>(fp, st);
-    case C6_PREC_BF16X2: return launch_forward<PrecBF16X2>(fp, st);
-    case C6_PREC_BF16F8: return launch_forward<PrecBF16F8>(fp, st);
     case C6_PREC_BF16F6: return launch_forward<PrecBF16F6>(fp, st);
   }
   set_error("unknown precision mode %d", prec);
   return C6_EINVAL;
-#endif
 }
 
 __global__ void cascade_reset_kernel(int *count) {
@@ -2317,8 +2144,6 @@ size_t packed_bytes(int prec) {
     case C6_PREC_F32: return Geo<PrecF32>::PACKED_BYTES;
     case C6_PREC_BF16: return Geo<PrecBF16>::PACKED_BYTES;
     case C6_PREC_F16: return Geo<PrecF16>::PACKED_BYTES;
-    case C6_PREC_BF16X2: return Geo<PrecBF16X2>::PACKED_BYTES;
-    case C6_PREC_BF16F8: return Geo<PrecBF16F8>::PACKED_BYTES;
     case C6_PREC_BF16F6: return Geo<PrecBF16F6>::PACKED_BYTES;
   }
   return 0;

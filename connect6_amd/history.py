@@ -35,12 +35,14 @@ def _normalized_model_cfg(cfg: dict[str, Any]) -> dict[str, Any]:
     return out
 
 
-# bfloat16 selects the corrected bf16 mode (bf16 MFMA + fp6 pass on what the activations'
-# rounding dropped), the fastest bf16 mode that keeps >= 99 % of the fp32 argmax; the literal
-# "round every activation to bf16" arithmetic stays available as precision="bf16".
+# bfloat16 selects the cascade (plain bf16 layer boundaries, then the boards whose decision is
+# close again with the fp6 pass on what the activations' rounding dropped), the fastest bf16 mode
+# that keeps the corrected arithmetic's agreement with the fp32 argmax; the literal "round every
+# activation to bf16" arithmetic stays available as precision="bf16", the correction on every
+# board as precision="bf16f6".
 _PREC_OF_DTYPE = {
     torch.float32: _lib.PREC_F32,
-    torch.bfloat16: _lib.PREC_BF16F6,
+    torch.bfloat16: _lib.PREC_BF16C,
     torch.float16: _lib.PREC_F16,
 }
 
@@ -66,9 +68,9 @@ class HistoricalPolicyEnsemble:
     Input ``[MODELS, TABLES, 3, H, W]`` -> policy logits ``[MODELS, TABLES,
     H*W]`` in the ensemble dtype.  ``dtype`` selects the arithmetic as in the
     reference's ``_history_dtype`` (connect6/train.py:133-145): float32,
-    bfloat16 or float16.  bfloat16 runs the corrected bf16 arithmetic
-    (``"bf16f6"``); ``precision`` may name any other mode, e.g. ``"bf16"``
-    for the literal bf16 rounding of every activation.
+    bfloat16 or float16.  bfloat16 runs the cascade (``"bf16c"``);
+    ``precision`` may name any other mode, e.g. ``"bf16"`` for the literal
+    bf16 rounding of every activation.
 
     ``conv_weights``, ``conv_biases``, ``policy_weight`` and ``policy_bias``
     (the reference's stacked ``[M, ...]`` tensors, connect6/history.py:224-233)
@@ -113,7 +115,7 @@ class HistoricalPolicyEnsemble:
         self.action_size = self.board_size * self.board_size
 
         self._prec = _PREC_OF_DTYPE[self.dtype] if precision is None else _lib.PREC_BY_NAME[precision]
-        self._packed: torch.Tensor | None = None
+        self._packed: tuple | None = None   # (buffer, stream it was packed on, event)
         self._states = states
         self._stacked: dict[str, torch.Tensor | None] = {}
 
@@ -167,13 +169,20 @@ class HistoricalPolicyEnsemble:
         return {k: src[k].detach().to(device=self.device, dtype=self.dtype) for k in keys if k in src}
 
     def _packed_weights(self) -> torch.Tensor:
+        stream = torch.cuda.current_stream(self.device)
         if self._packed is None:
             one = _lib.packed_bytes(self._prec)
             buf = torch.empty((self.num_models, one), dtype=torch.uint8, device=self.device)
             for m in range(self.num_models):
                 pack_state(self._model_state(m), self._prec, buf[m])
-            self._packed = buf
-        return self._packed
+            done = torch.cuda.Event()
+            done.record(stream)
+            self._packed = (buf, stream.cuda_stream, done)
+        buf, packed_on, done = self._packed
+        if packed_on != stream.cuda_stream:   # packed on another stream: wait for it, and tell the
+            stream.wait_event(done)           # allocator that this stream reads the buffer too
+            buf.record_stream(stream)
+        return buf
 
     def forward_grouped(self, x: torch.Tensor) -> torch.Tensor:
         if x.ndim != 5:

@@ -234,14 +234,19 @@ class PolicyValueNet(nn.Module):
 
     ``precision`` selects the arithmetic of the HIP path: ``None`` follows
     PyTorch's own rules (bf16/fp16 under ``torch.autocast`` or when the
-    parameters are held in that dtype, else fp32), where bf16 means
-    ``"bf16f6"``: bf16 MFMA whose result keeps at least 99 % of the fp32
-    argmax.  ``"bf16"`` (every activation rounded to bf16 and nothing else,
-    98.8-98.9 % agreement) has to be asked for by name.  Or one of ``"fp32"``,
-    ``"bf16"``, ``"fp16"``, ``"bf16x2"`` (bf16 MFMA with activations carried
-    as a hi+lo bf16 pair), ``"bf16f8"`` / ``"bf16f6"`` (bf16 MFMA plus a
-    correction pass on the activations' low-order part held in fp8 / in
-    block-scaled fp6).
+    parameters are held in that dtype, else fp32), where bf16 means the
+    cascade ``"bf16c"``: every board with plain bf16 layer boundaries, then
+    the boards whose best free square leads the second best by less than
+    ``cascade_threshold`` (default ``CASCADE_THRESHOLD`` = 0.03) standard
+    deviations of their logits once more with the corrected arithmetic.  It
+    keeps the corrected mode's agreement with the fp32 argmax (99.2 % in the
+    mean over random networks, a few of which fall just under 99 %) while
+    3-10 % of the boards of such networks are evaluated twice (all of them
+    when a network's logits are nearly flat).  The modes it is made of have
+    to be asked for by name: ``"bf16"`` (every activation rounded to bf16
+    and nothing else, 98.8-98.9 % agreement) and ``"bf16f6"`` (bf16 MFMA plus
+    a correction pass on the activations' low-order part held in
+    block-scaled fp6, on every board); also ``"fp32"`` and ``"fp16"``.
     """
 
     DEFAULT_KERNELS = (23, 3, 3, 3, 3, 3, 3, 3)
@@ -328,8 +333,8 @@ class PolicyValueNet(nn.Module):
         if torch.is_autocast_enabled("cuda"):  # reference: train.py:126-130 wraps calls in autocast
             dtype = torch.get_autocast_dtype("cuda")
         if dtype == torch.bfloat16:
-            # the corrected bf16 mode: plain "bf16" misses the 99 % argmax agreement with fp32
-            return _lib.PREC_BF16F6
+            # the cascade: plain "bf16" alone misses the 99 % argmax agreement with fp32
+            return _lib.PREC_BF16C
         if dtype == torch.float16:
             return _lib.PREC_F16
         return _lib.PREC_F32
@@ -357,6 +362,9 @@ class PolicyValueNet(nn.Module):
             _, buf, packed_on, done = hit
             if packed_on != stream.cuda_stream:
                 stream.wait_event(done)  # the pack kernel ran on another stream
+                # ... whose allocator owns the buffer: a repack drops it, and without this note the
+                # memory could be handed out again while a forward here still reads it
+                buf.record_stream(stream)
             return buf
         buf = torch.empty(_lib.packed_bytes(prec), dtype=torch.uint8, device=dev)
         pack_state({k: v for k, v in self.state_dict().items()}, prec, buf)

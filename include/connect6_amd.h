@@ -34,13 +34,10 @@ extern "C" {
 #define C6_PREC_F32 0    /* fp32 operands, fp32 MFMA                                        */
 #define C6_PREC_BF16 1   /* bf16 operands, bf16 MFMA, fp32 accumulate, bf16 layer boundaries */
 #define C6_PREC_F16 2    /* fp16 operands, fp16 MFMA, fp32 accumulate, fp16 layer boundaries */
-#define C6_PREC_BF16X2 3 /* bf16 MFMA, activations carried as a bf16 hi+lo pair (two passes)  */
-#define C6_PREC_BF16F8 4 /* bf16 MFMA + a second pass on the activations' dropped low-order
-                            part held as scaled fp8 (e4m3), on the fp8 MFMA at twice the rate */
-#define C6_PREC_BF16F6 5 /* the same with the low-order part held as block-scaled fp6 (e2m3,
-                            one power-of-two scale per 32 channels), at four times the rate */
-
-#define C6_PREC_BF16C 6  /* cascade: every board in C6_PREC_BF16, then the boards whose decision
+#define C6_PREC_BF16F6 3 /* bf16 MFMA + a second pass on what the bf16 rounding of each activation
+                            dropped, held as block-scaled fp6 (e2m3, one power-of-two scale per 32
+                            channels), on the fp6 MFMA at four times the bf16 rate */
+#define C6_PREC_BF16C 4  /* cascade: every board in C6_PREC_BF16, then the boards whose decision
                             is closer than the rounding noise again in C6_PREC_BF16F6; needs a
                             workspace: c6_forward_cascade / c6_forward_boards_cascade */
 

@@ -12,6 +12,7 @@ from connect6_amd import _lib
 from connect6_amd.model import run_forward
 from connect6_amd.synthetic import gen_boards
 from oracle import cref
+from oracle import lowprec_ref as Q
 from oracle import torch_ref as R
 from tests.util import argmax_agreement, rel_l2
 
@@ -20,6 +21,11 @@ pytestmark = pytest.mark.gpu
 FP32_TOL = 1e-4
 BF16_TOL = 2e-2
 ARGMAX_MIN = 0.99
+# the bf16 + fp6 kernel against its emulation (measured 1.4e-4 / 5.4e-7) and against the forward
+# with bf16 weights (measured 2.2e-4 / 1.1e-6), with slack; the weights' rounding alone puts both
+# 4.0e-3 / 2.7e-5 away from fp32, and the plain bf16 kernel sits 4.5e-3 / 2.7e-5 from the latter
+EMUL_TOL = {"reference": 4e-4, "torch_default": 3e-6}
+BF16W_TOL = {"reference": 6e-4, "torch_default": 5e-6}
 
 
 def make_model(dev, state, precision=None):
@@ -70,7 +76,7 @@ def test_zero_input_known_answer(cuda):
     # reference init (zero biases) every logit and the value are exactly zero
     model = c6.PolicyValueNet(board_size=19).to(cuda)
     with torch.inference_mode():
-        for prec in (None, "bf16", "fp16", "bf16x2", "bf16f8", "bf16f6"):
+        for prec in (None, "bf16", "fp16", "bf16f6", "bf16c"):
             model.precision = prec
             logits, value = model(torch.zeros(3, 3, 19, 19, device=cuda))
             assert logits.shape == (3, 361) and value.shape == (3,)
@@ -87,7 +93,7 @@ def test_ragged_batches(cuda, batch):
     assert rel_l2(lg, lo) <= FP32_TOL and rel_l2(vg, vo) <= FP32_TOL
 
 
-@pytest.mark.parametrize("prec", ["bf16f6", "bf16", "fp16", "bf16f8"])
+@pytest.mark.parametrize("prec", ["bf16f6", "bf16", "fp16", "bf16c"])
 def test_16bit_modes_on_ragged_batches(cuda, prec):
     """A board's result does not depend on the batch around it: every prefix of a batch gives,
     bit for bit, the rows of the whole batch (workgroups with one board, with none, with a
@@ -118,7 +124,7 @@ def test_empty_batch(cuda):
 
 
 @pytest.mark.parametrize("init", ["reference", "torch_default"])
-@pytest.mark.parametrize("prec", ["bf16f6", "bf16f8", "bf16x2", "fp16", "bf16"])
+@pytest.mark.parametrize("prec", ["bf16c", "bf16f6", "fp16", "bf16"])
 def test_16bit_paths_match_fp32_oracle_b4096(cuda, oracle_cfg2, init, prec):
     x, legal, outs = oracle_cfg2
     st, lo, vo = outs[init]
@@ -175,12 +181,13 @@ def test_input_dtypes_and_autocast(cuda):
             l, v = model(x.to(cuda).to(dt))
             assert torch.equal(l, l32) and torch.equal(v, v32)
         with torch.autocast(device_type="cuda", dtype=torch.bfloat16):   # train.py:126-130, :791-794
-            # bf16 means the corrected bf16 mode; the literal one has to be named
-            assert model.resolve_precision() == _lib.PREC_BF16F6
+            # bf16 means the cascade (plain bf16, corrected where it matters); the literal mode
+            # and the everywhere-corrected one have to be named
+            assert model.resolve_precision() == _lib.PREC_BF16C
             la, _ = model(x.to(cuda))
         with torch.autocast(device_type="cuda", dtype=torch.float16):
             assert model.resolve_precision() == _lib.PREC_F16
-        model.precision = "bf16f6"
+        model.precision = "bf16c"
         lb, _ = model(x.to(cuda))
         model.precision = "bf16"
         assert model.resolve_precision() == _lib.PREC_BF16
@@ -212,7 +219,7 @@ def test_grad_mode_is_refused(cuda):
         model(torch.zeros(1, 3, 19, 19, device=cuda))
 
 
-@pytest.mark.parametrize("prec", [None, "bf16x2", "bf16f8", "bf16f6"])
+@pytest.mark.parametrize("prec", [None, "bf16c", "bf16f6"])
 def test_masking_is_bit_exact(cuda, prec):
     st = R.init_state(1234, "reference")
     x, legal = gen_boards(512, 200, 2025)
@@ -273,7 +280,7 @@ def _bf16_params(state):
     return {k: v.to(torch.bfloat16).float() for k, v in state.items()}
 
 
-@pytest.mark.parametrize("precision", [None, "bf16x2", "bf16f8", "bf16f6"])
+@pytest.mark.parametrize("precision", [None, "bf16c", "bf16f6"])
 def test_grouped_g8_bf16_cfg3(cuda, precision):
     """Each group against its single-model fp32 oracle at the 16-bit tolerances: rel-L2 and
     >= 99 % argmax on masked logits (the reference's grouped == individual invariant,
@@ -283,7 +290,7 @@ def test_grouped_g8_bf16_cfg3(cuda, precision):
     torch.set_num_threads(16)
     cps = _checkpoints(8)
     ens = c6.HistoricalPolicyEnsemble(cps, cuda, dtype=torch.bfloat16, precision=precision)
-    assert ens._prec == _lib.PREC_BY_NAME[precision or "bf16f6"]
+    assert ens._prec == _lib.PREC_BY_NAME[precision or "bf16c"]
     x, legal = gen_boards(4096, 200, 2025)
     xg, lg = x.view(8, 512, 3, 19, 19), legal.view(8, 512, 361)
     with torch.inference_mode():
@@ -371,7 +378,9 @@ def test_runs_on_the_callers_stream_and_accepts_strided_input(cuda):
         assert torch.equal(got, want) and torch.equal(vgot, vwant)
 
 
-@pytest.mark.parametrize("prec", ["bf16f6", "bf16f8", "bf16x2", "bf16"])
+@pytest.mark.parametrize("prec", ["bf16c", "bf16f6", "bf16", pytest.param("fp16", marks=pytest.mark.skip(
+    reason="fp16 layer boundaries hold at most 65504: on this deliberately huge network they overflow "
+           "to inf by design (documented for the fp16 mode); the bf16 modes are the ones that must stay finite"))])
 def test_large_activations_stay_finite(cuda, prec):
     # weights 6x larger per layer: activations reach the hundreds, far beyond what the fp8 low-order
     # plane can represent (its inputs are clamped, so accuracy degrades to bf16's, never to NaN)
@@ -383,7 +392,6 @@ def test_large_activations_stay_finite(cuda, prec):
         lo, vo = R.forward(st, x)
         lg, vg = make_model(cuda, st, prec)(x.to(cuda))
     assert torch.isfinite(lo).all()
-    # (fp16 is left out: its 65504 range overflows on this deliberately huge network by design)
     assert torch.isfinite(lg).all() and torch.isfinite(vg).all()
     assert rel_l2(lg, lo) <= 5e-2
 
@@ -398,7 +406,7 @@ def test_headline_mode_keeps_the_argmax_gate_on_other_weights(cuda, seed):
     with torch.inference_mode():
         model.precision = "fp32"
         want, _ = model.forward_masked(x.to(cuda))
-        for prec in ("bf16f6", "bf16f8"):
+        for prec in ("bf16f6", "bf16c"):
             model.precision = prec
             got, _ = model.forward_masked(x.to(cuda))
             agree = float((got.argmax(1) == want.argmax(1)).float().mean())
@@ -406,27 +414,119 @@ def test_headline_mode_keeps_the_argmax_gate_on_other_weights(cuda, seed):
             assert agree >= ARGMAX_MIN
 
 
-def test_headline_mode_agreement_over_sixteen_more_seeds(cuda):
-    """How wide the margin of the >= 99 % gate is: sixteen further weight samples (reference
-    initialisation, the benchmark's boards).  Random networks have nearly flat logits and a few
-    of them fall just under 99 % on their own (8 mantissa bits of the *weights* are what is left
-    after the activation correction), so the bound is on the mean and on the worst sample."""
-    x, _ = gen_boards(4096, 200, 2025)
-    xd = x.to(cuda)
-    agree = {"bf16f6": [], "bf16": []}
-    for seed in range(1000, 1016):
-        torch.manual_seed(seed)
-        model = c6.PolicyValueNet().to(cuda).eval()
-        with torch.inference_mode():
-            model.precision = "fp32"
-            want = model.forward_masked(xd)[0].argmax(1)
-            for prec in agree:
-                model.precision = prec
-                agree[prec].append(float((model.forward_masked(xd)[0].argmax(1) == want).float().mean()))
-    f6, plain = torch.tensor(agree["bf16f6"]), torch.tensor(agree["bf16"])
-    print(f"bf16f6 mean {f6.mean():.4f} worst {f6.min():.4f}; bf16 mean {plain.mean():.4f} worst {plain.min():.4f}")
-    assert f6.mean() >= ARGMAX_MIN + 0.001 and f6.min() >= 0.985
-    assert (f6 > plain).all()  # the correction helps on every sample
+def test_argmax_margin_over_32_seeds_two_inits_two_densities(cuda):
+    """How wide the margin of the >= 99 % gate is, as numbers the suite owns: 32 further weight
+    samples x both initialisations x the benchmark's boards (stones <= 200) and nearly empty
+    boards (stones <= 20, the hardest input), 4096 boards each, every 16-bit bf16 mode against
+    the fp32 kernel.  Random networks have nearly flat logits and a few of them fall just under
+    99 % on their own: what is left after the activation correction is the rounding of the
+    *weights* to 8 mantissa bits.  The bounds are what was measured, with a little slack; the
+    cascade must keep the corrected mode's agreement on every sample."""
+    boards = {st: gen_boards(4096, st, 2025 + st)[0].to(cuda) for st in (200, 20)}
+    modes = ("bf16c", "bf16f6", "bf16")
+    res = {(init, st, m): [] for init in ("reference", "torch_default") for st in boards for m in modes}
+    twice = {(init, st): [] for init in ("reference", "torch_default") for st in boards}
+    for init in ("reference", "torch_default"):
+        for seed in range(1000, 1032):
+            torch.manual_seed(seed)
+            model = c6.PolicyValueNet().to(cuda).eval()
+            if init == "torch_default":
+                for mod in model.modules():
+                    if isinstance(mod, torch.nn.Conv2d):
+                        mod.reset_parameters()
+                model.refresh_weights()
+            for st, xd in boards.items():
+                with torch.inference_mode():
+                    model.precision = "fp32"
+                    want = model.forward_masked(xd)[0].argmax(1)
+                    for m in modes:
+                        model.precision = m
+                        got = model.forward_masked(xd)[0].argmax(1)
+                        res[(init, st, m)].append(float((got == want).float().mean()))
+                        if m == "bf16c":
+                            twice[(init, st)].append(int(model.cascade_stats["second_pass"].item()) / 4096)
+    t = {k: torch.tensor(v) for k, v in res.items()}
+    for (init, st, m), v in t.items():
+        extra = ""
+        if m == "bf16c":
+            f = torch.tensor(twice[(init, st)])
+            extra = f"; evaluated twice: mean {f.mean():.3f} max {f.max():.3f}"
+        print(f"{init:14s} stones<={st:3d} {m:7s}: mean {v.mean():.4f} worst {v.min():.4f} "
+              f"under 99 %: {int((v < 0.99).sum())}/32{extra}")
+    for init in ("reference", "torch_default"):
+        for st in boards:
+            c, f6, plain = t[(init, st, "bf16c")], t[(init, st, "bf16f6")], t[(init, st, "bf16")]
+            # the cascade gives up next to nothing: in the mean under 0.05 %, on a single network at
+            # most 0.15 % (0.3 % on the flat-logit networks of PyTorch's default initialisation,
+            # where a quarter of the boards sit near the threshold)
+            assert bool((c >= f6 - (0.0015 if init == "reference" else 0.003)).all())
+            assert c.mean() >= f6.mean() - 0.0005
+            assert bool((f6 >= plain).all())               # the correction never hurts
+    ref200, ref20 = t[("reference", 200, "bf16c")], t[("reference", 20, "bf16c")]
+    td200, td20 = t[("torch_default", 200, "bf16c")], t[("torch_default", 20, "bf16c")]
+    assert ref200.mean() >= ARGMAX_MIN + 0.0015 and ref200.min() >= 0.985 and int((ref200 < 0.99).sum()) <= 5
+    assert ref20.mean() >= ARGMAX_MIN + 0.0005 and ref20.min() >= 0.965 and int((ref20 < 0.99).sum()) <= 9
+    assert td200.mean() >= ARGMAX_MIN + 0.003 and td200.min() >= 0.97 and int((td200 < 0.99).sum()) <= 5
+    assert td20.mean() >= ARGMAX_MIN + 0.005 and td20.min() >= 0.96 and int((td20 < 0.99).sum()) <= 4
+    assert t[("reference", 200, "bf16")].mean() < ARGMAX_MIN     # why plain bf16 is not the default
+    # what the cascade costs on networks with the reference's initialisation
+    assert torch.tensor(twice[("reference", 200)]).mean() <= 0.10
+
+
+@pytest.mark.parametrize("prec", ["bf16c", "bf16f6", "bf16", "fp16"])
+def test_16bit_input_tensors_through_the_pipelined_kernel(cuda, prec):
+    """bf16 / fp16 input tensors (what a caller under autocast or a bf16 ensemble hands over)
+    travel as 2-byte elements, one per LDS word, and are decoded there; the check for a constant
+    third plane looks at the element's own 16 bits only.  Values exact in both types: the result
+    must equal the fp32-input result bit for bit, in a batch and alone."""
+    st = R.init_state(31, "reference")
+    x, _ = gen_boards(90, 200, 19)
+    g = torch.Generator().manual_seed(2)
+    x = x.clone()
+    x[0::3, 2] = torch.randint(0, 9, (30, 19, 19), generator=g).float() / 8.0    # a varying third plane
+    x[1::3, 2] = 0.375                                                           # constant, neither 0 nor 1
+    model = make_model(cuda, st, prec)
+    with torch.inference_mode():
+        want, vwant = model(x.to(cuda))
+        for dt in (torch.bfloat16, torch.float16):
+            xd = x.to(cuda).to(dt)
+            got, vgot = model(xd)
+            assert torch.equal(got, want) and torch.equal(vgot, vwant), dt
+            for i in (0, 1, 2):                        # one board of each kind, alone
+                one, vone = model(xd[i:i + 1])
+                assert torch.equal(one[0], want[i]) and torch.equal(vone[0], vwant[i]), (dt, i)
+
+
+@pytest.mark.parametrize("init", ["reference", "torch_default"])
+def test_corrected_arithmetic_matches_its_emulation(cuda, init):
+    """The bf16 + fp6 mode against oracle.lowprec_ref.forward_bf16f6_emulated (bf16 weights and
+    layer inputs, block-scaled e2m3 low-order parts contracted with the e2m3 weight copy, fp32
+    accumulation and SiLU): what is left between the two is fp32 summation order and the hardware's
+    exp2 / reciprocal.  And against the plain forward with the kernel's bf16 weights: what is left
+    there is the e2m3 rounding of the correction itself, far below the distance to fp32 that the
+    weights' rounding alone causes.  A correction that is wrong on one layer fails both."""
+    torch.set_num_threads(16)
+    st = R.init_state(1234, init)
+    x, legal = gen_boards(1024, 200, 2025)
+    with torch.inference_mode():
+        lk, vk = make_model(cuda, st, "bf16f6")(x.to(cuda))
+        lk, vk = lk.cpu(), vk.cpu()
+        le, ve = Q.forward_bf16f6_emulated(st, x)
+        stq = {k: (v.to(torch.bfloat16).float() if k.startswith("convs.") and k.endswith("weight") else v)
+               for k, v in st.items()}
+        stq["convs.0.weight"] = (st["convs.0.weight"] * Q.ACT_SCALE).to(torch.bfloat16).float() / Q.ACT_SCALE
+        stq["convs.0.weight"][:, 2] = st["convs.0.weight"][:, 2]   # a constant third plane (every board here)
+        lw, vw = R.forward(stq, x)                                   # takes its weights unrounded
+        l32, _ = R.forward(st, x)
+        lp, _ = make_model(cuda, st, "bf16")(x.to(cuda))
+    e_emul, e_w, e_32, e_plain = rel_l2(lk, le), rel_l2(lk, lw), rel_l2(lk, l32), rel_l2(lp.cpu(), lw)
+    print(f"{init}: bf16f6 vs its emulation {e_emul:.2e}; vs bf16-weight forward {e_w:.2e} "
+          f"(plain bf16 kernel: {e_plain:.2e}); vs fp32 {e_32:.2e}")
+    assert e_emul <= EMUL_TOL[init]
+    assert e_w <= BF16W_TOL[init] and e_w <= 0.2 * e_plain
+    assert rel_l2(vk, ve) <= EMUL_TOL[init]
+    agree = argmax_agreement(R.mask_logits(lk, legal), R.mask_logits(le, legal))
+    assert agree >= 0.998
 
 
 def test_c_abi_from_a_plain_cpp_program(cuda):

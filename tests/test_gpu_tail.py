@@ -85,7 +85,7 @@ def test_sample_edge_cases(cuda):
     assert torch.allclose(lp.cpu(), torch.log(torch.tensor([1.0, 1.0, 0.5, 1 / 361])), atol=1e-5)
 
 
-@pytest.mark.parametrize("prec", ["bf16f6", "bf16x2"])
+@pytest.mark.parametrize("prec", ["bf16f6", "bf16c"])
 def test_fused_selfplay_step_cfg4(cuda, prec):
     """B=16384, stones 0..300: forward + mask + softmax + draw in one launch, in the headline
     arithmetic mode (the one the benchmark times) and in the hi+lo bf16 mode."""
@@ -145,7 +145,7 @@ def test_d4_reduce_matches_oracle(cuda):
     assert none is None and torch.equal(only, logits)
 
 
-@pytest.mark.parametrize("prec", ["bf16f6", "bf16x2"])
+@pytest.mark.parametrize("prec", ["bf16f6", "bf16c"])
 def test_d4_evaluation_cfg5(cuda, prec):
     st = R.init_state(1234, "reference")
     model = c6.PolicyValueNet().to(cuda).eval()

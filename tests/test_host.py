@@ -30,10 +30,10 @@ def test_fused_kernels_stay_within_their_scratch_budget():
     arithmetic mode (headline and plain 16-bit modes tight, the others a ceiling)."""
     usage = _lib.resource_usage()
     fused = {name: u for name, u in usage.items() if "fused_forward_kernel" in name or "fused_pipe_kernel" in name}
-    assert len(fused) == 6
+    assert len(fused) == 4
     # bytes per lane; the pipelined kernels (bf16f6, bf16, fp16) keep two layers' accumulators live
-    # and still spill next to nothing: per-lane addresses are recomputed per board, not kept
-    limit = {"PrecBF16F6": 0, "PrecBF16E": 0, "PrecF16": 0, "PrecBF16F8": 32, "PrecF32": 32, "PrecBF16X2": 160}
+    # and still spill nothing: per-lane addresses are recomputed per board, not kept
+    limit = {"PrecBF16F6": 0, "PrecBF16E": 0, "PrecF16": 0, "PrecF32": 32}
     seen = set()
     for name, u in fused.items():
         for tag, cap in limit.items():
@@ -69,14 +69,17 @@ def test_packed_sizes_follow_the_layout():
     fast1 = 23 * 3 + 8 + 4 * 3 * 4
     assert _lib.packed_bytes(_lib.PREC_BF16) == (frags(8) + fast1) * 1024 + tail
     assert _lib.packed_bytes(_lib.PREC_F16) == (frags(8) + fast1) * 1024 + tail
-    assert _lib.packed_bytes(_lib.PREC_BF16X2) == frags(8) * 1024 + tail
     assert _lib.packed_bytes(_lib.PREC_F32) == frags(4) * 1024 + tail
-    # bf16 + fp8: plus the e4m3 copy of the 3x3 layers (64-wide chunks, two 16-byte pieces per lane)
+    # bf16 + fp6: plus the e2m3 copy of the 3x3 layers (64-wide chunks, two fragments per chunk and
+    # cout tile: 16 bytes per lane, then 8 bytes per lane packed densely) and its over-read padding
     lo = 0
     for cin, cout in zip((32, 32, 64, 64, 64, 96, 96), (32, 64, 64, 64, 96, 96, 96)):
         lo += ((9 * cin // 32 + 1) // 2) * (cout // 32) * 2
-    assert _lib.packed_bytes(_lib.PREC_BF16F8) == (frags(8) + lo + 18) * 1024 + tail
-    assert _lib.packed_bytes(_lib.PREC_BF16F6) == _lib.packed_bytes(_lib.PREC_BF16F8) + fast1 * 1024
+    assert _lib.packed_bytes(_lib.PREC_BF16F6) == (frags(8) + lo + 18 + fast1) * 1024 + tail
+    # cascade: the bf16 set, then (256-byte aligned) the bf16 + fp6 set
+    first = (_lib.packed_bytes(_lib.PREC_BF16) + 255) // 256 * 256
+    assert _lib.packed_bytes(_lib.PREC_BF16C) == first + _lib.packed_bytes(_lib.PREC_BF16F6)
+    assert _lib.cascade_workspace_bytes(0) == 16 and _lib.cascade_workspace_bytes(5) == 48
     with pytest.raises(ValueError):
         _lib.packed_bytes(9)
 
@@ -90,6 +93,19 @@ def test_entry_points_reject_bad_arguments_before_touching_the_device():
     assert lib.c6_forward(None, 0, 0, 4, None, 0, 1, None, None, 0, None, 0.0, None, 1.0, None, None, None) == -1
     # an empty batch is a no-op, not an error
     assert lib.c6_forward(None, 0, 1, 0, None, 0, 1, None, None, 0, None, 0.0, None, 1.0, None, None, None) == 0
+    # the cascade's mode only through the entry points that take its workspace, and those only it
+    assert lib.c6_forward(None, 0, 1, 4, None, 0, _lib.PREC_BF16C, None, None, 0, None, 0.0, None, 1.0, None, None,
+                          None) == -1
+    assert b"c6_forward_cascade" in lib.c6_last_error()
+    assert lib.c6_forward_cascade(None, 0, 1, 4, None, 0, None, None, 0, None, 0.0, None, 1.0, None, None, 0.03,
+                                  None, 0, None) == -1
+    assert lib.c6_forward_cascade(None, 0, 1, 0, None, 0, None, None, 0, None, 0.0, None, 1.0, None, None, 0.03,
+                                  None, 0, None) == 0
+    assert lib.c6_forward_boards_cascade(None, None, None, 4, None, 0, 4, None, None, None, 1, 0.0, None, 1.0,
+                                         None, None, 0.03, None, 0, None) == -1
+    size = ctypes.c_size_t(0)
+    assert lib.c6_cascade_workspace_bytes(-1, ctypes.byref(size)) == -1
+    assert lib.c6_cascade_workspace_bytes(4096, ctypes.byref(size)) == 0 and size.value == 16 + 4 * 4096
     assert lib.c6_mask_logits(None, None, 0, 3, 0, None, None) == -1
     assert lib.c6_mask_logits(None, None, 0, 0, 0, None, None) == 0
     assert lib.c6_softmax_sample(None, None, None, 1.0, 2, None, None, None) == -1
@@ -196,11 +212,12 @@ def test_forward_errors():
 def test_precision_resolution_follows_torch_rules():
     model = c6.PolicyValueNet()
     assert model.resolve_precision() == _lib.PREC_F32
-    model.precision = "bf16x2"
-    assert model.resolve_precision() == _lib.PREC_BF16X2
+    model.precision = "bf16f6"
+    assert model.resolve_precision() == _lib.PREC_BF16F6
     model.precision = None
-    # bf16 parameters (or bf16 autocast) select the corrected bf16 mode; plain bf16 is by name only
-    assert model.to(torch.bfloat16).resolve_precision() == _lib.PREC_BF16F6
+    # bf16 parameters (or bf16 autocast) select the cascade (plain bf16, corrected where the
+    # decision is close); the two modes it is made of are by name only
+    assert model.to(torch.bfloat16).resolve_precision() == _lib.PREC_BF16C
     assert model.to(torch.float16).resolve_precision() == _lib.PREC_F16
     model.precision = "bf16"
     assert model.resolve_precision() == _lib.PREC_BF16
@@ -235,7 +252,7 @@ def test_history_ensemble_construction_and_validation():
     assert ens.policy_weight.shape == (2, 1, 96, 1, 1) and ens.policy_bias.shape == (2, 1)
     assert ens._prec == _lib.PREC_F32
     ens16 = c6.HistoricalPolicyEnsemble(cps, torch.device("cpu"), dtype=torch.bfloat16)
-    assert ens16._prec == _lib.PREC_BF16F6 and ens16.conv_weights[3].dtype == torch.bfloat16
+    assert ens16._prec == _lib.PREC_BF16C and ens16.conv_weights[3].dtype == torch.bfloat16
     assert c6.HistoricalPolicyEnsemble(cps, torch.device("cpu"), dtype=torch.bfloat16, precision="bf16")._prec == _lib.PREC_BF16
     # compile keys are ignored when comparing architectures (history.py:69-73)
     cps[1].model_config["compile"] = True
