@@ -214,8 +214,15 @@ def main() -> int:
         ens128 = c6.HistoricalPolicyEnsemble(cps128, dev, dtype=torch.bfloat16,
                                              precision=None if args.precision == "fp32" else args.precision)
         xg128 = x[:512].view(128, 4, 3, 19, 19).to(torch.bfloat16)
+        ens128.conv_weights, ens128.conv_biases, ens128.policy_weight, ens128.policy_bias   # (stack: host work + H2D)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        ens128._packed_weights()                 # 128 weight sets into kernel layout: two launches
+        torch.cuda.synchronize()
+        pack128 = time.perf_counter() - t0
         tg128 = timed(lambda: ens128.forward_grouped(xg128))
-        out["grouped_g128x4"] = {"boards_per_s": 512 / tg128, "ms": tg128 * 1e3}
+        out["grouped_g128x4"] = {"boards_per_s": 512 / tg128, "ms": tg128 * 1e3,
+                                 "pack_128_weight_sets_ms": pack128 * 1e3}
         del ens128, cps128
 
         # ---- fused self-play step, configs[3]: B=16384, stones 0..300 ----

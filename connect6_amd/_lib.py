@@ -23,8 +23,11 @@ _RESOURCES = _LIBDIR / "resource_usage.txt"   # registers, scratch and LDS of ev
 PREC_F32, PREC_BF16, PREC_F16, PREC_BF16F6, PREC_BF16C = 0, 1, 2, 3, 4
 PREC_BY_NAME = {"fp32": PREC_F32, "bf16": PREC_BF16, "fp16": PREC_F16, "bf16f6": PREC_BF16F6, "bf16c": PREC_BF16C}
 # cascade mode: a board is evaluated a second time (corrected arithmetic) when its best free
-# square leads the second best by less than this many standard deviations of its logits
-CASCADE_THRESHOLD = 0.03
+# square leads the second best by less than this many standard deviations of its logits, or two
+# other free squares lie within twice that.  The plain pass's error on a difference of two logits
+# has a standard deviation of about 0.01 standard deviations of the logits: the threshold is two
+# of those.
+CASCADE_THRESHOLD = 0.02
 DT_F32, DT_BF16, DT_F16 = 0, 1, 2
 MASK_NONE, MASK_INPUT, MASK_LEGAL = 0, 1, 2
 
@@ -34,6 +37,7 @@ EXPORTS = (
     "c6_last_error",
     "c6_packed_bytes",
     "c6_pack_weights",
+    "c6_pack_weights_grouped",
     "c6_forward",
     "c6_forward_boards",
     "c6_cascade_workspace_bytes",
@@ -175,10 +179,13 @@ def load() -> ctypes.CDLL:
     lib.c6_cascade_workspace_bytes.restype = i32
     lib.c6_cascade_workspace_bytes.argtypes = [i64, ctypes.POINTER(ctypes.c_size_t)]
     lib.c6_forward_cascade.restype = i32
-    lib.c6_forward_cascade.argtypes = [vp, i32, i64, i64, vp, ctypes.c_size_t, vp, vp, i32, vp, f32,
+    lib.c6_pack_weights_grouped.restype = i32
+    lib.c6_pack_weights_grouped.argtypes = [ctypes.POINTER(vp), ctypes.POINTER(vp), vp, vp, vp, vp, i64, i32, vp,
+                                            ctypes.c_size_t, vp]
+    lib.c6_forward_cascade.argtypes = [vp, i32, i64, i64, vp, ctypes.c_size_t, vp, i32, vp, i32, vp, f32,
                                        vp, f32, vp, vp, f32, vp, ctypes.c_size_t, vp]
     lib.c6_forward_boards_cascade.restype = i32
-    lib.c6_forward_boards_cascade.argtypes = [vp, vp, vp, i64, vp, i32, i64, vp, vp, vp, i32, f32, vp, f32,
+    lib.c6_forward_boards_cascade.argtypes = [vp, vp, vp, i64, vp, i32, i64, vp, vp, i32, vp, i32, f32, vp, f32,
                                               vp, vp, f32, vp, ctypes.c_size_t, vp]
     ip = ctypes.POINTER(ctypes.c_int)
     lib.c6_generic_workspace_bytes.restype = i32

@@ -109,19 +109,25 @@ int c6_packed_bytes(int prec, size_t *bytes) {
   return C6_OK;
 }
 
-int c6_pack_weights(const float *const *conv_w, const float *const *conv_b, const float *pol_w,
-                    const float *pol_b, const float *val_w, const float *val_b, int prec,
-                    void *packed, void *stream) {
+int c6_pack_weights_grouped(const float *const *conv_w, const float *const *conv_b,
+                            const float *pol_w, const float *pol_b, const float *val_w,
+                            const float *val_b, int64_t groups, int prec, void *packed,
+                            size_t packed_stride, void *stream) {
   if (!valid_prec(prec)) {
     set_error("c6_pack_weights: unknown precision mode %d", prec);
+    return C6_EINVAL;
+  }
+  if (groups < 1 || groups > 65535) {
+    set_error("c6_pack_weights: %lld weight sets (one call packs 1 to 65535)", (long long)groups);
     return C6_EINVAL;
   }
   if (conv_w == nullptr || pol_w == nullptr || packed == nullptr) {
     set_error("c6_pack_weights: conv_w, pol_w and packed must not be null");
     return C6_EINVAL;
   }
-  if (!aligned16(packed)) {
-    set_error("c6_pack_weights: packed buffer must be 16-byte aligned");
+  if (!aligned16(packed) || (packed_stride & 15u) != 0 || (groups > 1 && packed_stride < packed_bytes(prec))) {
+    set_error("c6_pack_weights: packed buffer must be 16-byte aligned, its sets a multiple of 16 "
+              "bytes and at least c6_packed_bytes() apart");
     return C6_EINVAL;
   }
   PackParams pp;
@@ -138,14 +144,22 @@ int c6_pack_weights(const float *const *conv_w, const float *const *conv_b, cons
   pp.val_w = val_w;
   pp.val_b = val_b;
   pp.packed = static_cast<unsigned char *>(packed);
+  pp.groups = (int)groups;
+  pp.packed_stride = packed_stride;
   C6_REQUIRE_DEVICE("c6_pack_weights");
   return dispatch_pack(prec, pp, static_cast<hipStream_t>(stream));
+}
+
+int c6_pack_weights(const float *const *conv_w, const float *const *conv_b, const float *pol_w,
+                    const float *pol_b, const float *val_w, const float *val_b, int prec,
+                    void *packed, void *stream) {
+  return c6_pack_weights_grouped(conv_w, conv_b, pol_w, pol_b, val_w, val_b, 1, prec, packed, 0, stream);
 }
 
 // c6_forward and c6_forward_cascade (workspace != nullptr: the latter)
 static int forward_planes(const char *who, const void *x, int x_dtype, int64_t groups,
                           int64_t boards_per_group, const void *packed, size_t packed_stride,
-                          int prec, float *logits, float *value, int mask_mode,
+                          int prec, void *logits, int logits_dtype, float *value, int mask_mode,
                           const uint8_t *legal, float fill, const float *u, float temperature,
                           int64_t *actions, float *logprob, bool cascade, float threshold,
                           void *workspace, size_t workspace_bytes, void *stream) {
@@ -154,8 +168,8 @@ static int forward_planes(const char *who, const void *x, int x_dtype, int64_t g
               "takes c6_forward_cascade, every other mode c6_forward)", who, prec);
     return C6_EINVAL;
   }
-  if (elem_bytes(x_dtype) == 0) {
-    set_error("%s: unknown input element type %d", who, x_dtype);
+  if (elem_bytes(x_dtype) == 0 || elem_bytes(logits_dtype) == 0) {
+    set_error("%s: unknown element type of the input (%d) or of the logits (%d)", who, x_dtype, logits_dtype);
     return C6_EINVAL;
   }
   if (groups < 1 || boards_per_group < 0) {
@@ -195,6 +209,7 @@ static int forward_planes(const char *who, const void *x, int x_dtype, int64_t g
   fp.packed = static_cast<const unsigned char *>(packed);
   fp.packed_stride = packed_stride;
   fp.logits = logits;
+  fp.logits_dtype = logits_dtype;
   fp.value = value;
   fp.mask_mode = mask_mode;
   fp.legal = legal;
@@ -222,7 +237,7 @@ int c6_forward(const void *x, int x_dtype, int64_t groups, int64_t boards_per_gr
                int mask_mode, const uint8_t *legal, float fill, const float *u, float temperature,
                int64_t *actions, float *logprob, void *stream) {
   return forward_planes("c6_forward", x, x_dtype, groups, boards_per_group, packed, packed_stride, prec,
-                        logits, value, mask_mode, legal, fill, u, temperature, actions, logprob, false,
+                        logits, C6_DT_F32, value, mask_mode, legal, fill, u, temperature, actions, logprob, false,
                         0.0f, nullptr, 0, stream);
 }
 
@@ -236,23 +251,24 @@ int c6_cascade_workspace_bytes(int64_t boards, size_t *bytes) {
 }
 
 int c6_forward_cascade(const void *x, int x_dtype, int64_t groups, int64_t boards_per_group,
-                       const void *packed, size_t packed_stride, float *logits, float *value,
+                       const void *packed, size_t packed_stride, void *logits, int logits_dtype, float *value,
                        int mask_mode, const uint8_t *legal, float fill, const float *u,
                        float temperature, int64_t *actions, float *logprob, float threshold,
                        void *workspace, size_t workspace_bytes, void *stream) {
   return forward_planes("c6_forward_cascade", x, x_dtype, groups, boards_per_group, packed, packed_stride,
-                        C6_PREC_BF16C, logits, value, mask_mode, legal, fill, u, temperature, actions,
-                        logprob, true, threshold, workspace, workspace_bytes, stream);
+                        C6_PREC_BF16C, logits, logits_dtype, value, mask_mode, legal, fill, u, temperature,
+                        actions, logprob, true, threshold, workspace, workspace_bytes, stream);
 }
 
 
 static int forward_states(const char *who, const int8_t *boards, const int8_t *player,
                           const int8_t *stones_left, int64_t num_states, const int64_t *index,
-                          int view, int64_t batch, const void *packed, int prec, float *logits,
-                          float *value, int mask_mode, float fill, const float *u,
+                          int view, int64_t batch, const void *packed, int prec, void *logits,
+                          int logits_dtype, float *value, int mask_mode, float fill, const float *u,
                           float temperature, int64_t *actions, float *logprob, bool cascade,
                           float threshold, void *workspace, size_t workspace_bytes, void *stream) {
-  if (!valid_prec(prec) || (prec == C6_PREC_BF16C) != cascade || batch < 0 || batch > 0x7fffffffLL || view < 0 || view > 7 || num_states < 0) {
+  if (!valid_prec(prec) || (prec == C6_PREC_BF16C) != cascade || elem_bytes(logits_dtype) == 0 || batch < 0 ||
+      batch > 0x7fffffffLL || view < 0 || view > 7 || num_states < 0) {
     set_error("%s: bad precision %d, batch %lld, states %lld or view %d", who, prec,
               (long long)batch, (long long)num_states, view);
     return C6_EINVAL;
@@ -287,6 +303,7 @@ static int forward_states(const char *who, const int8_t *boards, const int8_t *p
   fp.packed = static_cast<const unsigned char *>(packed);
   fp.packed_stride = 0;
   fp.logits = logits;
+  fp.logits_dtype = logits_dtype;
   fp.value = value;
   fp.mask_mode = mask_mode;
   fp.legal = nullptr;
@@ -315,20 +332,20 @@ int c6_forward_boards(const int8_t *boards, const int8_t *player, const int8_t *
                       float *logits, float *value, int mask_mode, float fill, const float *u,
                       float temperature, int64_t *actions, float *logprob, void *stream) {
   return forward_states("c6_forward_boards", boards, player, stones_left, num_states, index, view, batch,
-                        packed, prec, logits, value, mask_mode, fill, u, temperature, actions, logprob,
+                        packed, prec, logits, C6_DT_F32, value, mask_mode, fill, u, temperature, actions, logprob,
                         false, 0.0f, nullptr, 0, stream);
 }
 
 int c6_forward_boards_cascade(const int8_t *boards, const int8_t *player,
                               const int8_t *stones_left, int64_t num_states,
                               const int64_t *index, int view, int64_t batch, const void *packed,
-                              float *logits, float *value, int mask_mode, float fill,
+                              void *logits, int logits_dtype, float *value, int mask_mode, float fill,
                               const float *u, float temperature, int64_t *actions,
                               float *logprob, float threshold, void *workspace,
                               size_t workspace_bytes, void *stream) {
   return forward_states("c6_forward_boards_cascade", boards, player, stones_left, num_states, index, view,
-                        batch, packed, C6_PREC_BF16C, logits, value, mask_mode, fill, u, temperature,
-                        actions, logprob, true, threshold, workspace, workspace_bytes, stream);
+                        batch, packed, C6_PREC_BF16C, logits, logits_dtype, value, mask_mode, fill, u,
+                        temperature, actions, logprob, true, threshold, workspace, workspace_bytes, stream);
 }
 
 

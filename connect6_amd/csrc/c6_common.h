@@ -86,7 +86,11 @@ struct PrecBF16F6 {
   // the reference's initialisation / with PyTorch's default one) all layers give 99.23 / 99.55 %,
   // without the last layer 99.17 / 93.3 %, without the last two 99.07 / 93.0 %, without layers 2
   // and 3 99.10 / 99.56 %: flat-logit networks need the late layers, the others every layer.
-  static constexpr int LO_MASK = 0xfe;
+  // (connect6_amd/profiling.py builds copies with other masks to price the layers one by one)
+#ifndef C6_LO_MASK
+#define C6_LO_MASK 0xfe
+#endif
+  static constexpr int LO_MASK = C6_LO_MASK;
 };
 
 // bf16 + fp6 mode: what rounding an activation to bf16 drops (|lo| <= 2^-9 |a|) is contracted
@@ -208,7 +212,8 @@ struct FwdParams {
   long long boards_per_group;
   const unsigned char *packed;
   size_t packed_stride;
-  float *logits;
+  void *logits;               // [boards, 361] of element type logits_dtype (fp32 unless the caller says so)
+  int logits_dtype = C6_DT_F32;
   float *value;
   int mask_mode;
   const uint8_t *legal;
@@ -231,10 +236,12 @@ struct FwdParams {
 };
 
 struct PackParams {
-  const float *conv_w[8];
+  const float *conv_w[8];     // each tensor stacked over the weight sets: [groups, ...]
   const float *conv_b[8];
   const float *pol_w, *pol_b, *val_w, *val_b;
   unsigned char *packed;
+  int groups = 1;             // weight sets (at most 65535: one grid row each)
+  size_t packed_stride = 0;   // bytes between consecutive packed sets
 };
 
 // state and results of VectorConnect6.step (connect6/vector_env.py:33-53, :8-14 of the reference)

@@ -73,36 +73,40 @@ __device__ __forceinline__ float wave_min(float v) {
   }));
 }
 
-// Does the largest of a board's 361 logits (entries with ok(i) only) lead the second largest by
-// less than `tau` standard deviations of those logits?  One wave; tau < 0 answers yes for every
-// board, and a board with fewer than two such entries has no margin to judge: no.
-// Everything is taken relative to the largest logit, so a large common offset of the logits
-// (flat policies) costs no precision.
+// Is the decision of a board (the largest of its 361 logits, entries with ok(i) only) closer than
+// the rounding noise of the plain bf16 pass?  Yes when the largest logit leads the second largest
+// by less than `tau` standard deviations of those logits, or when at least two other logits lie
+// within 2 tau standard deviations of it (several near-ties multiply the chance that one of them
+// overtakes).  One wave; tau < 0 answers yes for every board, and a board with fewer than two
+// such entries has no decision to judge: no.  Everything is taken relative to the largest logit,
+// so a large common offset of the logits (flat policies) costs no precision.
 template <class FZ, class FOK>
 __device__ __forceinline__ bool wave_margin_below(int lane, float tau, FZ z, FOK ok) {
   constexpr int PER = 6;  // 64 lanes x 6 = 384 >= 361
-  float v[PER];
+  float d[PER];           // largest - logit (>= 0), inf for entries that do not count
   float m = -INFINITY;
   int n = 0;
 #pragma unroll
   for (int e = 0; e < PER; ++e) {
     const int i = lane * PER + e;
     const bool use = (i < kPix) && ok(i);
-    v[e] = use ? z(i) : -INFINITY;
-    m = fmaxf(m, v[e]);
+    d[e] = use ? z(i) : -INFINITY;
+    m = fmaxf(m, d[e]);
     n += use ? 1 : 0;
   }
   m = wave_max(m);
-  // d = largest - logit >= 0: the margin is the second smallest d (the smallest is 0)
+  // the margin is the second smallest d (the smallest is 0)
   float d1 = INFINITY, d2 = INFINITY, s = 0.0f, ss = 0.0f;
 #pragma unroll
   for (int e = 0; e < PER; ++e) {
-    if (v[e] != -INFINITY) {
-      const float d = m - v[e];
-      s += d;
-      ss = fmaf(d, d, ss);
-      d2 = d < d1 ? d1 : fminf(d2, d);
-      d1 = fminf(d1, d);
+    if (d[e] != -INFINITY) {
+      d[e] = m - d[e];
+      s += d[e];
+      ss = fmaf(d[e], d[e], ss);
+      d2 = d[e] < d1 ? d1 : fminf(d2, d[e]);
+      d1 = fminf(d1, d[e]);
+    } else {
+      d[e] = INFINITY;
     }
   }
   const float cnt = wave_sum((float)n);
@@ -117,7 +121,12 @@ __device__ __forceinline__ bool wave_margin_below(int lane, float tau, FZ z, FOK
   if (tau < 0.0f) return true;
   const float mean = s / cnt;
   const float var = fmaxf(ss / cnt - mean * mean, 0.0f);
-  return gap * gap < tau * tau * var;
+  const float t2 = tau * tau * var;
+  int near = 0;  // entries within 2 tau standard deviations of the largest (itself included)
+#pragma unroll
+  for (int e = 0; e < PER; ++e) near += (d[e] * d[e] < 4.0f * t2) ? 1 : 0;
+  const float nearf = wave_sum((float)near);
+  return gap * gap < t2 || nearf >= 3.0f;
 }
 
 // Masked softmax + inverse-CDF draw over 361 entries by ONE wave.

@@ -1096,6 +1096,11 @@ __device__ __forceinline__ void pipe_layer(
     });
   }
   C6_MARK(4 + 2 * L);
+#ifdef C6_IDLE_PER_LAYER
+  // (profiling builds only: idle cycles with no work attached, to see how the card's power
+  // management trades them against the shader clock; s_sleep counts in units of 64 cycles)
+  __builtin_amdgcn_s_sleep(C6_IDLE_PER_LAYER);
+#endif
   (void)wave;
   (void)trace_on;
 }
@@ -1540,8 +1545,15 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
     // ---- write out: masked logits, optional sampled action ----
     if (prm.logits != nullptr) {
       for (int p = tidv; p < kPix; p += THREADS) {
-        const float v = lgt[p];
-        prm.logits[(size_t)b * kPix + p] = (occ[p] & 1) ? prm.fill : v;
+        const float v = (occ[p] & 1) ? prm.fill : lgt[p];
+        const size_t at = (size_t)b * kPix + p;
+        if (prm.logits_dtype == C6_DT_F32) {
+          static_cast<float *>(prm.logits)[at] = v;
+        } else if (prm.logits_dtype == C6_DT_BF16) {  // (round to nearest even, as Tensor.to does)
+          static_cast<unsigned short *>(prm.logits)[at] = __builtin_bit_cast(unsigned short, (__bf16)v);
+        } else {
+          static_cast<unsigned short *>(prm.logits)[at] = __builtin_bit_cast(unsigned short, (_Float16)v);
+        }
       }
     }
     if (prm.actions != nullptr && wave == 0) {
@@ -1805,7 +1817,7 @@ __global__ __launch_bounds__(256) void fused_forward_kernel(const FwdParams prm)
     if (prm.logits != nullptr) {
       for (int p = tid; p < kPix; p += THREADS) {
         const float v = lgt[p];
-        prm.logits[(size_t)b * kPix + p] = occ[p] ? prm.fill : v;
+        static_cast<float *>(prm.logits)[(size_t)b * kPix + p] = occ[p] ? prm.fill : v;
       }
     }
     if (prm.actions != nullptr && wave == 0) {
@@ -1844,9 +1856,32 @@ template <class P> __device__ __forceinline__ void put_elem(unsigned char *dst, 
   }
 }
 
+// The parameters of weight set `g` of a (possibly stacked) PackParams.
+struct GroupView {
+  const PackParams &p;
+  int g;
+  unsigned char *packed;
+  const float *pol_w, *pol_b, *val_w, *val_b;
+  __device__ GroupView(const PackParams &pp, int group)
+      : p(pp), g(group), packed(pp.packed + (size_t)group * pp.packed_stride),
+        pol_w(pp.pol_w + (size_t)group * kHeadC), pol_b(pp.pol_b ? pp.pol_b + group : nullptr),
+        val_w(pp.val_w ? pp.val_w + (size_t)group * kHeadC : nullptr),
+        val_b(pp.val_b ? pp.val_b + group : nullptr) {}
+  __device__ const float *conv_w(int l) const {
+    const int k = l == 0 ? kK1 : 3;
+    return p.conv_w[l] + (size_t)g * kCoutArr[l] * kCinArr[l] * k * k;
+  }
+  __device__ const float *conv_b(int l) const {
+    return p.conv_b[l] ? p.conv_b[l] + (size_t)g * kCoutArr[l] : nullptr;
+  }
+};
+
 // one thread per (fragment, lane): writes the 16 bytes that lane will load
-template <class P> __global__ void pack_kernel(const PackParams prm) {
+// (blockIdx.y = weight set: the parameter tensors are stacked [sets, ...], the packed sets lie
+// packed_stride bytes apart)
+template <class P> __global__ void pack_kernel(const PackParams all) {
   using G = Geo<P>;
+  const GroupView prm(all, blockIdx.y);
   const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   const long long nfl = (long long)G::TOTAL_FRAGS * 64;
   if (gid < nfl) {
@@ -1866,7 +1901,7 @@ template <class P> __global__ void pack_kernel(const PackParams prm) {
         const int r = p / kBoard, c = p % kBoard;
         f32x4 t4;
         for (int e = 0; e < 4; ++e) {
-          const float *w = prm.conv_w[0] + (size_t)((8 * q + 4 * h + e) * 3 + 2) * kK1 * kK1;
+          const float *w = prm.conv_w(0) + (size_t)((8 * q + 4 * h + e) * 3 + 2) * kK1 * kK1;
           float sum = 0.0f;
           for (int ky = 0; ky < kK1; ++ky) {
             const int rr = r + ky - kK1 / 2;
@@ -1884,7 +1919,7 @@ template <class P> __global__ void pack_kernel(const PackParams prm) {
       if (G::FAST1_FRAGS > 0 && frag >= G::FAST1_OFF && frag < G::FAST1_OFF + G::FAST1_STEPS) {
         // k-step (ky, 8 columns); lane half = input plane
         const int fi = frag - G::FAST1_OFF, ky = fi / G::CPR, jj = fi % G::CPR;
-        const float *w = prm.conv_w[0];
+        const float *w = prm.conv_w(0);
         for (int e = 0; e < G::E; ++e) {
           const int kx = jj * G::E + e;
           put_elem<P>(dst, e, kx < kK1 ? w[((m * 3 + h) * kK1 + ky) * kK1 + kx] * act_scale<P>() : 0.0f);
@@ -1901,7 +1936,7 @@ template <class P> __global__ void pack_kernel(const PackParams prm) {
           const int g = 2 * c + h;
           if (g < G::lo_half_chunks(ll)) {
             const int tap = g / per32, cb = g % per32, co = 32 * t + m;
-            const float *w = prm.conv_w[ll];
+            const float *w = prm.conv_w(ll);
             const float sc = exp2f((float)reinterpret_cast<const int *>(prm.packed + G::TAIL_OFF)[G::TAIL_SW + ll]);
             // the lane's 32 K slots as e2m3 (the copy approximates the bf16 weights the main pass
             // uses): 24 bytes = piece 0 + piece 1
@@ -1938,7 +1973,7 @@ template <class P> __global__ void pack_kernel(const PackParams prm) {
     const int nt = cout / 32;
     const int s = fi / nt, t = fi - s * nt;
     const int co = 32 * t + m;
-    const float *w = prm.conv_w[l];
+    const float *w = prm.conv_w(l);
     if (l == 0) {
       const int row = s / G::CPR + kL1RowsHalf * h;  // (ky, plane) row, 69 real + 1 pad
       const int jj = s % G::CPR;
@@ -1981,7 +2016,7 @@ template <class P> __global__ void pack_kernel(const PackParams prm) {
     if (ti < kBiasTotal) {
       int l = 0;
       while (ti >= bias_offset(l + 1)) ++l;
-      v = prm.conv_b[l] ? prm.conv_b[l][ti - bias_offset(l)] * act_scale<P>() : 0.0f;
+      v = prm.conv_b(l) ? prm.conv_b(l)[ti - bias_offset(l)] * act_scale<P>() : 0.0f;
     } else if (ti < kBiasTotal + kHeadC) {
       v = prm.pol_w[ti - kBiasTotal] / act_scale<P>();
     } else if (ti < kBiasTotal + 2 * kHeadC) {
@@ -1997,8 +2032,9 @@ template <class P> __global__ void pack_kernel(const PackParams prm) {
 
 // sw[l] = largest power of two that keeps 2^sw * max|w_l| inside the range of the low-order
 // weight copy's format (one block per layer)
-template <class P> __global__ __launch_bounds__(256) void lo_scale_kernel(const PackParams prm) {
+template <class P> __global__ __launch_bounds__(256) void lo_scale_kernel(const PackParams all) {
   using G = Geo<P>;
+  const GroupView prm(all, blockIdx.y);
   __shared__ float red[256];
   const int l = blockIdx.x;
   int *sw = reinterpret_cast<int *>(prm.packed + G::TAIL_OFF) + G::TAIL_SW;
@@ -2008,7 +2044,7 @@ template <class P> __global__ __launch_bounds__(256) void lo_scale_kernel(const 
   }
   const int n = kCoutArr[l] * kCinArr[l] * 9;
   float m = 0.0f;
-  for (int i = threadIdx.x; i < n; i += blockDim.x) m = fmaxf(m, fabsf(prm.conv_w[l][i]));
+  for (int i = threadIdx.x; i < n; i += blockDim.x) m = fmaxf(m, fabsf(prm.conv_w(l)[i]));
   red[threadIdx.x] = m;
   __syncthreads();
   for (int s = 128; s > 0; s >>= 1) {
@@ -2031,8 +2067,9 @@ template <class P> static int launch_pack(const PackParams &pp, hipStream_t st) 
   const long long total = (long long)G::TOTAL_FRAGS * 64 + G::TAIL_FLOATS;
   const int threads = 256;
   const int blocks = (int)((total + threads - 1) / threads);
-  if constexpr (P::LO6) hipLaunchKernelGGL(lo_scale_kernel<P>, dim3(8), dim3(256), 0, st, pp);
-  hipLaunchKernelGGL(pack_kernel<P>, dim3(blocks), dim3(threads), 0, st, pp);
+  const unsigned sets = (unsigned)pp.groups;
+  if constexpr (P::LO6) hipLaunchKernelGGL(lo_scale_kernel<P>, dim3(8, sets), dim3(256), 0, st, pp);
+  hipLaunchKernelGGL(pack_kernel<P>, dim3(blocks, sets), dim3(threads), 0, st, pp);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     set_error("pack_kernel launch failed: %s", hipGetErrorString(e));

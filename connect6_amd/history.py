@@ -173,8 +173,12 @@ class HistoricalPolicyEnsemble:
         if self._packed is None:
             one = _lib.packed_bytes(self._prec)
             buf = torch.empty((self.num_models, one), dtype=torch.uint8, device=self.device)
-            for m in range(self.num_models):
-                pack_state(self._model_state(m), self._prec, buf[m])
+            # one call for all models, from the stacked tensors (rounded to `dtype`, as the
+            # ensemble holds its parameters): two launches, however many models
+            keys = [f"convs.{i}.{kind}" for i in range(len(self.kernels)) for kind in ("weight", "bias")]
+            keys += ["policy_output.weight", "policy_output.bias"]
+            stacked = {k: self._stacked_attr(k, optional=k.endswith("bias")) for k in keys}
+            pack_state(stacked, self._prec, buf, groups=self.num_models)
             done = torch.cuda.Event()
             done.record(stream)
             self._packed = (buf, stream.cuda_stream, done)
@@ -205,8 +209,11 @@ class HistoricalPolicyEnsemble:
         if t == 0:
             return torch.empty((m, 0, self.action_size), dtype=self.dtype, device=self.device)
         if self.is_default_architecture:
+            # (the cascade's entry point writes the logits in the ensemble's type itself)
+            direct = self._prec == _lib.PREC_BF16C and self.dtype != torch.float32
             logits, _, _, _ = run_forward(x.reshape(m * t, *expected_tail), self._packed_weights(),
-                                          self._prec, m, t, want_value=False)
+                                          self._prec, m, t, want_value=False,
+                                          logits_dtype=self.dtype if direct else torch.float32)
         else:  # other architectures: layer by layer, one model after the other
             logits = torch.cat([
                 run_forward_generic(x[i], self._model_state(i), self.kernels, self.channels,

@@ -27,14 +27,19 @@ def _require_device_tensor(t: torch.Tensor, what: str) -> None:
         )
 
 
-def pack_state(state: dict[str, torch.Tensor], prec: int, out: torch.Tensor) -> None:
+def pack_state(state: dict[str, torch.Tensor], prec: int, out: torch.Tensor, groups: int | None = None) -> None:
     """Repack one checkpoint (reference ``state_dict`` keys, device tensors)
-    into ``out`` (uint8 device buffer of ``_lib.packed_bytes(prec)`` bytes)."""
+    into ``out`` (uint8 device buffer of ``_lib.packed_bytes(prec)`` bytes).
+
+    With ``groups`` = G every tensor of ``state`` is G checkpoints' tensors stacked along a
+    new first dimension (what ``HistoricalPolicyEnsemble._stack`` builds) and ``out`` is
+    ``[G, packed_bytes]``: all sets are packed by one call."""
     lib = _lib.load()
     keep = []  # keep fp32 staging copies alive until the launch is enqueued
+    lead = () if groups is None else (int(groups),)
 
     def dev32(key: str, required: bool = True):
-        if key not in state:
+        if key not in state or state[key] is None:
             if required:
                 raise KeyError(f"missing parameter {key}")
             return None
@@ -46,10 +51,10 @@ def pack_state(state: dict[str, torch.Tensor], prec: int, out: torch.Tensor) -> 
     bs = [dev32(f"convs.{i}.bias", required=False) for i in range(8)]
     expect_in = 3
     for i, (k, c) in enumerate(zip(PolicyValueNet.DEFAULT_KERNELS, PolicyValueNet.DEFAULT_CHANNELS)):
-        if tuple(ws[i].shape) != (c, expect_in, k, k):
+        if tuple(ws[i].shape) != lead + (c, expect_in, k, k):
             raise ValueError(
                 f"convs.{i}.weight has shape {tuple(ws[i].shape)}; the fused kernels are built for "
-                f"the default architecture and need {(c, expect_in, k, k)}"
+                f"the default architecture and need {lead + (c, expect_in, k, k)}"
             )
         expect_in = c
     pw, pb = dev32("policy_output.weight"), dev32("policy_output.bias", required=False)
@@ -62,8 +67,14 @@ def pack_state(state: dict[str, torch.Tensor], prec: int, out: torch.Tensor) -> 
         return t.data_ptr() if t is not None else None
 
     with torch.cuda.device(out.device):
-        rc = lib.c6_pack_weights(wptrs, bptrs, ptr(pw), ptr(pb), ptr(vw), ptr(vb), prec,
-                                 out.data_ptr(), _lib.stream_ptr(out.device))
+        if groups is None:
+            rc = lib.c6_pack_weights(wptrs, bptrs, ptr(pw), ptr(pb), ptr(vw), ptr(vb), prec,
+                                     out.data_ptr(), _lib.stream_ptr(out.device))
+        else:
+            if out.ndim != 2 or out.shape[0] != groups or not out.is_contiguous():
+                raise ValueError(f"out must be a contiguous [{groups}, packed_bytes] buffer")
+            rc = lib.c6_pack_weights_grouped(wptrs, bptrs, ptr(pw), ptr(pb), ptr(vw), ptr(vb), int(groups), prec,
+                                             out.data_ptr(), int(out.shape[1]), _lib.stream_ptr(out.device))
     _lib.check(rc, "c6_pack_weights")
     # the staging copies are freed by the caching allocator in stream order, after the kernel
 
@@ -85,16 +96,21 @@ def run_forward(
     want_logprob: bool = False,
     threshold: float | None = None,
     stats: dict | None = None,
+    logits_dtype: torch.dtype = torch.float32,
 ):
     """Launch ``c6_forward`` (``c6_forward_cascade`` for the cascade mode, with ``threshold``
     and a workspace tensor of its own); returns (logits, value, actions, logprob), each None
     when not requested.  ``stats``, if given, receives ``second_pass`` for the cascade mode: a
-    one-element int32 device tensor, the number of boards that were evaluated twice."""
+    one-element int32 device tensor, the number of boards that were evaluated twice.
+    ``logits_dtype`` other than float32 (the cascade mode's entry point only) makes the kernel
+    write the logits rounded to that type."""
     lib = _lib.load()
     dev = x.device
     total = groups * boards_per_group
     x = x.contiguous()
-    logits = torch.empty((total, 361), dtype=torch.float32, device=dev) if want_logits else None
+    if logits_dtype != torch.float32 and prec != _lib.PREC_BF16C:
+        raise ValueError("only the cascade mode's entry point writes logits in another type than float32")
+    logits = torch.empty((total, 361), dtype=logits_dtype, device=dev) if want_logits else None
     value = torch.empty((total,), dtype=torch.float32, device=dev) if want_value else None
     actions = logprob = None
     if u is not None:
@@ -122,8 +138,9 @@ def run_forward(
             ws = torch.empty(_lib.cascade_workspace_bytes(total) // 4, dtype=torch.int32, device=dev)
             rc = lib.c6_forward_cascade(
                 x.data_ptr(), _lib.torch_dtype_code(x.dtype), groups, boards_per_group, packed.data_ptr(),
-                stride, ptr(logits), ptr(value), mask_mode, ptr(legal), fill, ptr(u), float(temperature),
-                ptr(actions), ptr(logprob), float(_lib.CASCADE_THRESHOLD if threshold is None else threshold),
+                stride, ptr(logits), _lib.torch_dtype_code(logits_dtype), ptr(value), mask_mode, ptr(legal), fill,
+                ptr(u), float(temperature), ptr(actions), ptr(logprob),
+                float(_lib.CASCADE_THRESHOLD if threshold is None else threshold),
                 ws.data_ptr(), ws.numel() * 4, _lib.stream_ptr(dev))
             if stats is not None:
                 stats["second_pass"] = ws[:1]
@@ -236,13 +253,15 @@ class PolicyValueNet(nn.Module):
     PyTorch's own rules (bf16/fp16 under ``torch.autocast`` or when the
     parameters are held in that dtype, else fp32), where bf16 means the
     cascade ``"bf16c"``: every board with plain bf16 layer boundaries, then
-    the boards whose best free square leads the second best by less than
-    ``cascade_threshold`` (default ``CASCADE_THRESHOLD`` = 0.03) standard
-    deviations of their logits once more with the corrected arithmetic.  It
-    keeps the corrected mode's agreement with the fp32 argmax (99.2 % in the
-    mean over random networks, a few of which fall just under 99 %) while
-    3-10 % of the boards of such networks are evaluated twice (all of them
-    when a network's logits are nearly flat).  The modes it is made of have
+    the boards whose decision is closer than that pass's rounding noise (the
+    best free square leads the second best by less than ``cascade_threshold``
+    standard deviations of the board's logits, default ``CASCADE_THRESHOLD``
+    = 0.02, or two others lie within twice that) once more with the corrected
+    arithmetic.  Over random networks it keeps the corrected mode's agreement
+    with the fp32 argmax to 0.01-0.02 % in the mean (99.2 %; a few such
+    networks fall just under 99 % in either mode) while about 6 % of their
+    boards are evaluated twice (a quarter, or all, when a network's logits
+    are nearly flat).  The modes it is made of have
     to be asked for by name: ``"bf16"`` (every activation rounded to bf16
     and nothing else, 98.8-98.9 % agreement) and ``"bf16f6"`` (bf16 MFMA plus
     a correction pass on the activations' low-order part held in
@@ -570,7 +589,7 @@ def _forward_boards(
             thr = _lib.CASCADE_THRESHOLD if model.cascade_threshold is None else model.cascade_threshold
             rc = _lib.load().c6_forward_boards_cascade(
                 boards.data_ptr(), current_player.data_ptr(), stones_left.data_ptr(), n, ptr(index),
-                int(view), b, packed.data_ptr(), ptr(logits), value.data_ptr(),
+                int(view), b, packed.data_ptr(), ptr(logits), _lib.DT_F32, value.data_ptr(),
                 _lib.MASK_INPUT if masked else _lib.MASK_NONE,
                 _FILL_LOWEST if fill is None else float(fill), ptr(u), float(temperature),
                 ptr(actions), ptr(logprob), float(thr), ws.data_ptr(), ws.numel() * 4, _lib.stream_ptr(dev))

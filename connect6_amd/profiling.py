@@ -6,6 +6,15 @@ boundaries of the third board of every workgroup); ``python -m connect6_amd.prof
 then runs B=4096 forwards on the GPU through that copy and prints, per arithmetic mode, the mean
 cycles per phase over all workgroups and waves and the shader clock during the traced board.
 The shipped library contains none of this.
+
+``python -m connect6_amd.profiling --threshold-sweep`` (the ordinary library) prints, for a range
+of cascade thresholds, how many boards are evaluated twice and what that costs in argmax agreement
+with the fp32 kernel, over 32 random networks of either initialisation.
+
+``python -m connect6_amd.profiling --build-ablations`` compiles further traced copies (the
+corrected mode without the low-order pass of some layers; with idle cycles added) and
+``python -m connect6_amd.profiling --ablations`` measures them back to back: cycles per board, shader
+clock, time per launch, agreement with fp32.
 """
 from __future__ import annotations
 
@@ -28,15 +37,94 @@ _PIPE_NAMES = ["stage input", "conv1 K-loop"] + sum(
       f"conv{l + 1} low-order pass", f"conv{l + 1} last phase (parts A, B)"] for l in range(1, 8)], []) + ["heads", "write out"]
 
 
-def build_traced() -> Path:
+def _traced_build_command(out: Path, defines=()) -> list[str]:
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc, "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-DC6_TRACE",
-           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-function",
-           "-o", str(TRACE_SO)] + [str(_lib._CSRC / s) for s in _lib._SOURCES]
-    proc = subprocess.run(cmd, capture_output=True, text=True)
+    return ([hipcc, "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-DC6_TRACE"]
+            + [f"-D{d}" for d in defines]
+            + ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-function",
+               "-o", str(out)] + [str(_lib._CSRC / s) for s in _lib._SOURCES])
+
+
+def build_traced() -> Path:
+    proc = subprocess.run(_traced_build_command(TRACE_SO), capture_output=True, text=True)
     if proc.returncode != 0:
         raise _lib.C6Error(f"hipcc failed ({proc.returncode}):\n{proc.stderr[-4000:]}")
     return TRACE_SO
+
+
+# Ablation copies of the traced library: the corrected mode ("bf16f6") with the low-order pass of
+# some layers left out (their results then differ: these price the layers, they are not modes),
+# and with idle cycles added at every layer end.  name -> (what it is, extra compiler defines)
+ABLATIONS = {
+    "all": ("low-order pass on the input of every 3x3 layer (the library as shipped)", ()),
+    "no8": ("without the last layer's", ("C6_LO_MASK=0x7e",)),
+    "no78": ("without the last two layers'", ("C6_LO_MASK=0x3e",)),
+    "no678": ("without the last three layers'", ("C6_LO_MASK=0x1e",)),
+    "no23": ("without layers 2 and 3", ("C6_LO_MASK=0xf8",)),
+    "none": ("no low-order pass, no low-order part computed (bf16 arithmetic in this mode's record layout)",
+             ("C6_LO_MASK=0x00",)),
+    "idle": ("every layer, plus 40 x 64 idle cycles at the end of each 3x3 layer", ("C6_IDLE_PER_LAYER=40",)),
+}
+
+
+def _ablation_so(name: str) -> Path:
+    return TRACE_SO if name == "all" else _lib._LIBDIR / f"libconnect6_amd_trace_{name}.so"
+
+
+def build_ablations(jobs: int = 4) -> list[Path]:
+    """Compile every ablation copy (``jobs`` compilers at a time; each takes a few minutes)."""
+    pending = [(n, subprocess.Popen(_traced_build_command(_ablation_so(n), ABLATIONS[n][1]), stdout=subprocess.PIPE,
+                                    stderr=subprocess.PIPE, text=True)) for n in list(ABLATIONS)[:jobs]]
+    todo = list(ABLATIONS)[jobs:]
+    built = []
+    while pending:
+        name, proc = pending.pop(0)
+        _, err = proc.communicate()
+        if proc.returncode != 0:
+            raise _lib.C6Error(f"hipcc failed for ablation {name} ({proc.returncode}):\n{err[-4000:]}")
+        built.append(_ablation_so(name))
+        if todo:
+            n = todo.pop(0)
+            pending.append((n, subprocess.Popen(_traced_build_command(_ablation_so(n), ABLATIONS[n][1]),
+                                                stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)))
+    return built
+
+
+def ablation_row(name: str, batch: int = 4096, launches: int = 150) -> str:
+    """One row of the ablation table, measured in this process (which must not have loaded the
+    library yet): cycles per board and shader clock from the traced board, time per launch from
+    HIP events over the last 20 launches, argmax agreement with the fp32 kernel."""
+    import numpy as np
+    import torch
+
+    global TRACE_SO
+    TRACE_SO = _ablation_so(name)
+    table = phase_table("bf16f6", batch=batch, launches=launches)
+    head = table.splitlines()[0]
+    import connect6_amd as c6
+    from connect6_amd.synthetic import gen_boards
+
+    dev = torch.device("cuda:0")
+    torch.manual_seed(1234)
+    model = c6.PolicyValueNet().to(dev).eval()
+    x = gen_boards(batch, 200, 2025)[0].to(dev)
+    with torch.inference_mode():
+        model.precision = "fp32"
+        want = model.forward_masked(x)[0].argmax(1)
+        model.precision = "bf16f6"
+        got = model.forward_masked(x)[0].argmax(1)
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(20)]
+        for a, b in evs:
+            a.record()
+            model.forward_masked(x)
+            b.record()
+        torch.cuda.synchronize()
+    ms = float(np.mean([a.elapsed_time(b) for a, b in evs]))
+    cycles = head.split("one board = ")[1].split(" shader")[0]
+    clock = head.rsplit(" at ", 1)[1]
+    agree = float((got == want).float().mean())
+    return (f"| {name} | {ABLATIONS[name][0]} | {cycles} | {clock} | {ms:.4f} | "
+            f"{batch * 269554368 / (ms * 1e-3) / 2.5e15 * 100:.1f} | {agree:.4f} |")
 
 
 def phase_table(precision: str, batch: int = 4096, launches: int = 150) -> str:
@@ -85,9 +173,79 @@ def phase_table(precision: str, batch: int = 4096, launches: int = 150) -> str:
     return "\n".join(lines)
 
 
+def threshold_sweep(thresholds=(0.01, 0.015, 0.02, 0.025, 0.03, 0.04), seeds=range(1000, 1032), batch: int = 4096) -> str:
+    """Cascade mode: boards evaluated twice and argmax agreement with the fp32 kernel per
+    threshold, against the corrected mode on every board (bf16f6) and plain bf16."""
+    import torch
+
+    import connect6_amd as c6
+    from connect6_amd.synthetic import gen_boards
+
+    dev = torch.device("cuda:0")
+    lines = []
+    for stones in (200, 20):
+        x = gen_boards(batch, stones, 2025 + stones)[0].to(dev)
+        for init in ("reference", "torch_default"):
+            acc = {t: [] for t in thresholds}
+            frac = {t: [] for t in thresholds}
+            fine, plain = [], []
+            for seed in seeds:
+                torch.manual_seed(seed)
+                m = c6.PolicyValueNet().to(dev).eval()
+                if init == "torch_default":
+                    for mod in m.modules():
+                        if isinstance(mod, torch.nn.Conv2d):
+                            mod.reset_parameters()
+                    m.refresh_weights()
+                with torch.inference_mode():
+                    m.precision = "fp32"
+                    want = m.forward_masked(x)[0].argmax(1)
+                    agree = lambda: float((m.forward_masked(x)[0].argmax(1) == want).float().mean())
+                    m.precision = "bf16f6"
+                    fine.append(agree())
+                    m.precision = "bf16"
+                    plain.append(agree())
+                    m.precision = "bf16c"
+                    for t in thresholds:
+                        m.cascade_threshold = t
+                        acc[t].append(agree())
+                        frac[t].append(int(m.cascade_stats["second_pass"].item()) / batch)
+            f6 = torch.tensor(fine)
+            lines += [f"stones <= {stones}, {init} initialisation, {len(fine)} networks x {batch} boards: "
+                      f"bf16f6 {f6.mean():.4f}, bf16 {torch.tensor(plain).mean():.4f} (mean argmax agreement with fp32)",
+                      "", "| threshold | evaluated twice, mean (max) | agreement, mean | vs bf16f6, mean | worst network | networks losing > 0.1 % |",
+                      "|---|---|---|---|---|---|"]
+            for t in thresholds:
+                a, f = torch.tensor(acc[t]), torch.tensor(frac[t])
+                d = a - f6
+                lines.append(f"| {t:g} | {f.mean():.3f} ({f.max():.3f}) | {a.mean():.4f} | {d.mean():+.5f} | {d.min():+.4f} | "
+                             f"{int((d < -0.001).sum())} / {len(fine)} |")
+            lines.append("")
+    return "\n".join(lines)
+
+
 def main(argv: list[str]) -> int:
     if argv and argv[0] == "--build":
         print(build_traced())
+        return 0
+    if argv and argv[0] == "--threshold-sweep":
+        print(threshold_sweep())
+        return 0
+    if argv and argv[0] == "--build-ablations":
+        for so in build_ablations():
+            print(so)
+        return 0
+    if argv and argv[0] == "--ablation-row":
+        print(ablation_row(argv[1]))
+        return 0
+    if argv and argv[0] == "--ablations":
+        print("| build | low-order passes | cycles per board | shader clock | ms per 4096 boards | % of 2.5 PFLOP/s | argmax agreement with fp32 |")
+        print("|---|---|---|---|---|---|---|")
+        for name in ABLATIONS:   # one process per copy: each must be the first library the process loads
+            out = subprocess.run([sys.executable, "-m", "connect6_amd.profiling", "--ablation-row", name],
+                                 capture_output=True, text=True)
+            print(out.stdout.strip().splitlines()[-1] if out.returncode == 0 and out.stdout.strip() else
+                  f"| {name} | failed: {out.stderr[-300:]!r} | | | | | |")
         return 0
     for i, prec in enumerate(argv or ["bf16f6"]):
         if i:   # one process per mode keeps every run the library's first use

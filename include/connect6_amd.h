@@ -72,6 +72,17 @@ int c6_pack_weights(const float *const *conv_w, const float *const *conv_b,
                     const float *pol_w, const float *pol_b, const float *val_w,
                     const float *val_b, int prec, void *packed, void *stream);
 
+/* The same for `groups` checkpoints in one call (two launches whatever their number): every
+ * parameter tensor is the checkpoints' tensors stacked along a new first dimension, as
+ * HistoricalPolicyEnsemble._stack builds them (connect6/history.py:224-240): conv_w[i] device fp32
+ * [groups,Cout,Cin,k,k], conv_b[i] [groups,Cout], pol_w / val_w [groups,1,96,1,1], pol_b / val_b
+ * [groups,1].  Set g is written at packed + g * packed_stride (a multiple of 16 bytes, at least
+ * c6_packed_bytes(prec)); 1 <= groups <= 65535. */
+int c6_pack_weights_grouped(const float *const *conv_w, const float *const *conv_b,
+                            const float *pol_w, const float *pol_b, const float *val_w,
+                            const float *val_b, int64_t groups, int prec, void *packed,
+                            size_t packed_stride, void *stream);
+
 /* Batched forward of G weight sets, each applied to T boards, in one launch.
  * Replaces: PolicyValueNet.forward (connect6/model.py:96-111) with G = 1, and
  * HistoricalPolicyEnsemble.forward_grouped (connect6/history.py:276-303) with
@@ -119,28 +130,34 @@ int c6_forward_boards(const int8_t *boards, const int8_t *player, const int8_t *
  * for that mode).  Replaces the same reference calls as they do (connect6/model.py:96-111,
  * connect6/history.py:276-303, connect6/train.py:730-748, :791-799).
  * First every board is evaluated with plain bf16 layer boundaries.  A board is evaluated again,
- * with the low-order correction of C6_PREC_BF16F6, when its largest logit among the free squares
+ * with the low-order correction of C6_PREC_BF16F6, when the rounding of the plain pass can change
+ * the move that an argmax picks (reference callers: connect6/benchmark.py:32,44,
+ * connect6/evaluate.py:54, connect6/gui_cnn.py:43): when its largest logit among the free squares
  * (free as C6_MASK_LEGAL or the input planes say, whatever mask_mode writes) leads the second
- * largest by less than `threshold` standard deviations of the free squares' logits: that is
- * where the rounding of the plain pass can change the move that an argmax picks (reference
- * callers: connect6/benchmark.py:32,44, connect6/evaluate.py:54, connect6/gui_cnn.py:43).  Its
- * logits, value and draw replace the first ones.  threshold = 0 evaluates no board twice
- * (results of C6_PREC_BF16), threshold < 0 every board (results of C6_PREC_BF16F6); 0.03 keeps
- * the corrected mode's agreement with fp32 on random networks while 3-10 % of the boards are
- * evaluated twice.  A board's results do not depend on the other boards of the batch.
+ * largest by less than `threshold` standard deviations of the free squares' logits, or when two
+ * other free squares lie within twice that of the largest.  Its logits, value and draw replace
+ * the first ones.  threshold = 0 evaluates no board twice (results of C6_PREC_BF16), threshold < 0
+ * every board (results of C6_PREC_BF16F6).  The plain pass's error on a difference of two logits
+ * is about 0.01 standard deviations of the logits; with threshold 0.02 random networks lose
+ * 0.01-0.02 % of the corrected mode's agreement with fp32 in the mean while about 6 % of their
+ * boards are evaluated twice.  A board's results do not depend on the other boards of the batch.
+ *   logits     device [boards,361] of element type logits_dtype (C6_DT_F32, C6_DT_BF16 or
+ *              C6_DT_F16; may be NULL): a bf16 / fp16 ensemble gets its logits rounded once (to
+ *              nearest even, as Tensor.to does) by the kernel instead of by a cast behind it;
+ *              `fill` is converted the same way
  *   workspace  device, c6_cascade_workspace_bytes(boards) bytes, 16-byte aligned; after the
  *              call its first int32 holds the number of boards that were evaluated twice
  * Three launches on `stream`, no synchronisation with the host. */
 int c6_cascade_workspace_bytes(int64_t boards, size_t *bytes);
 int c6_forward_cascade(const void *x, int x_dtype, int64_t groups, int64_t boards_per_group,
-                       const void *packed, size_t packed_stride, float *logits, float *value,
-                       int mask_mode, const uint8_t *legal, float fill, const float *u,
+                       const void *packed, size_t packed_stride, void *logits, int logits_dtype,
+                       float *value, int mask_mode, const uint8_t *legal, float fill, const float *u,
                        float temperature, int64_t *actions, float *logprob, float threshold,
                        void *workspace, size_t workspace_bytes, void *stream);
 int c6_forward_boards_cascade(const int8_t *boards, const int8_t *player,
                               const int8_t *stones_left, int64_t num_states,
                               const int64_t *index, int view, int64_t batch, const void *packed,
-                              float *logits, float *value, int mask_mode, float fill,
+                              void *logits, int logits_dtype, float *value, int mask_mode, float fill,
                               const float *u, float temperature, int64_t *actions,
                               float *logprob, float threshold, void *workspace,
                               size_t workspace_bytes, void *stream);

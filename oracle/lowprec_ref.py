@@ -25,8 +25,8 @@ function                   pinned by (tests/test_oracle.py)
                            bit for bit; with exact (unquantised) low-order parts and weights it
                            equals the forward with bf16 weights and unrounded activations to
                            fp32 rounding; its distance to fp32 is below plain bf16's.
-``cascade_second_pass``    brute-force double-precision loop over the legal squares of small
-                           hand-made boards (ties, one legal square, flat logits).
+``cascade_margin`` /       brute-force double-precision loop over the legal squares of small
+``cascade_second_pass``    hand-made boards (ties, one or two legal squares, flat logits).
 =========================  ====================================================================
 """
 from __future__ import annotations
@@ -141,31 +141,36 @@ def forward_bf16f6_emulated(
     return logits, value
 
 
-def cascade_margin(logits: torch.Tensor, free: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
-    """Per board: (lead of the largest logit over the second largest, standard deviation of the
-    logits), both over the free squares only, in double precision.  Boards with fewer than two
-    free squares get (inf, 0)."""
+def cascade_margin(logits: torch.Tensor, free: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Per board, over the free squares only and in double precision: (lead of the largest logit
+    over the second largest, lead over the third largest, standard deviation of the logits).
+    Missing entries (fewer than two / three free squares) are inf, the deviation then 0."""
     z = logits.double()
     neg = torch.full_like(z, float("-inf"))
     zf = torch.where(free, z, neg)
-    top2 = zf.topk(2, dim=1).values
+    top3 = zf.topk(3, dim=1).values
     cnt = free.sum(dim=1)
-    gap = top2[:, 0] - top2[:, 1]
+    gap2 = top3[:, 0] - top3[:, 1]          # (inf where the second entry is a masked square)
+    gap3 = top3[:, 0] - top3[:, 2]
     zero = torch.zeros_like(z)
     mean = torch.where(free, z, zero).sum(1) / cnt.clamp_min(1)
     var = torch.where(free, (z - mean[:, None]) ** 2, zero).sum(1) / cnt.clamp_min(1)
     few = cnt < 2
-    gap = torch.where(few, torch.full_like(gap, float("inf")), gap)
+    inf = torch.full_like(gap2, float("inf"))
+    gap2 = torch.where(few, inf, gap2)
+    gap3 = torch.where(cnt < 3, inf, gap3)
     std = torch.where(few, torch.zeros_like(var), var.sqrt())
-    return gap, std
+    return gap2, gap3, std
 
 
 def cascade_second_pass(logits: torch.Tensor, free: torch.Tensor, threshold: float) -> torch.Tensor:
     """The cascade's rule: a board is evaluated a second time iff it has at least two free
-    squares and the lead of its best free square is below ``threshold`` standard deviations of
-    its free squares' logits (``threshold < 0``: every such board)."""
-    gap, std = cascade_margin(logits, free)
+    squares and either the lead of its best free square over the second best is below
+    ``threshold`` standard deviations of its free squares' logits, or at least two other free
+    squares (so also the third best) lie within twice that of the best.  ``threshold < 0``:
+    every board with two free squares."""
+    gap2, gap3, std = cascade_margin(logits, free)
     enough = free.sum(dim=1) >= 2
     if threshold < 0:
         return enough
-    return enough & (gap < threshold * std)
+    return enough & ((gap2 < threshold * std) | (gap3 < 2 * threshold * std))

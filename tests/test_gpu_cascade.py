@@ -75,12 +75,13 @@ def test_rows_follow_the_rule_and_keep_the_gates_b4096(cuda, init):
     from_f6 = (lc == lf).all(1) & (vc == vf)
     from_b = (lc == lb).all(1) & (vc == vb)
     assert bool((from_f6 | from_b).all())
-    # ... chosen by the rule, judged on the first pass's logits (boards within 2 % of the
+    # ... chosen by the rule, judged on the first pass's logits (boards within 2 % of a
     # threshold aside: the kernel sums in fp32 and in another order)
-    gap, std = Q.cascade_margin(lb, legal)
+    gap2, gap3, std = Q.cascade_margin(lb, legal)
     thr = _lib.CASCADE_THRESHOLD
     want = Q.cascade_second_pass(lb, legal, thr)
-    clear = (gap < 0.98 * thr * std) | (gap > 1.02 * thr * std)
+    near = lambda g, t: (g > 0.98 * t * std) & (g < 1.02 * t * std)
+    clear = ~(near(gap2, thr) | near(gap3, 2 * thr))
     took_second = from_f6 & ~from_b                    # (rows equal in both modes tell nothing)
     took_first = from_b & ~from_f6
     assert not bool((took_second & ~want & clear).any())
@@ -94,9 +95,9 @@ def test_rows_follow_the_rule_and_keep_the_gates_b4096(cuda, init):
     print(f"{init}: second pass {n2} of 4096 ({n2 / 4096:.3f}); argmax agreement cascade {agree:.4f}, "
           f"bf16f6 {agree_f6:.4f}, bf16 {argmax_agreement(masked(lb), masked(lo)):.4f}")
     assert agree >= ARGMAX_MIN
-    assert agree >= agree_f6 - 0.0015                  # what the threshold is allowed to cost
+    assert agree >= agree_f6 - 0.002                   # what the threshold is allowed to cost
     if init == "reference":
-        assert n2 <= 0.15 * 4096                       # the cascade pays: few boards go twice
+        assert n2 <= 0.10 * 4096                       # the cascade pays: few boards go twice
 
 
 def test_a_boards_result_does_not_depend_on_the_batch(cuda):
@@ -142,7 +143,7 @@ def test_grouped_sets_go_through_both_passes(cuda):
         grouped = ens.forward_grouped(xg.to(cuda))
         assert torch.equal(grouped, raw.view(8, 512, 361).to(torch.bfloat16))
         n2 = int(stats["second_pass"].item())
-        assert 0 < n2 < 0.15 * 4096
+        assert 0 < n2 < 0.10 * 4096
         raw = raw.view(8, 512, 361).cpu()
         for i, cp in enumerate(cps):
             st16 = {k: v.to(torch.bfloat16).float() for k, v in cp.model_state.items()}
@@ -164,7 +165,7 @@ def test_cascade_entry_points_check_their_workspace(cuda):
     x = gen_boards(100, 200, 1)[0].to(cuda)
     out = torch.empty(100, 361, device=cuda)
     small = torch.empty(16, dtype=torch.int32, device=cuda)
-    args = (x.data_ptr(), _lib.DT_F32, 1, 100, packed.data_ptr(), packed.numel(), out.data_ptr(), None,
+    args = (x.data_ptr(), _lib.DT_F32, 1, 100, packed.data_ptr(), packed.numel(), out.data_ptr(), _lib.DT_F32, None,
             _lib.MASK_NONE, None, 0.0, None, 1.0, None, None, 0.03)
     rc = lib.c6_forward_cascade(*args, small.data_ptr(), small.numel() * 4, _lib.stream_ptr(cuda))
     assert rc == -1 and b"workspace" in lib.c6_last_error()
@@ -174,3 +175,34 @@ def test_cascade_entry_points_check_their_workspace(cuda):
     rc = lib.c6_forward(x.data_ptr(), _lib.DT_F32, 1, 100, packed.data_ptr(), packed.numel(), _lib.PREC_BF16C,
                         out.data_ptr(), None, _lib.MASK_NONE, None, 0.0, None, 1.0, None, None, _lib.stream_ptr(cuda))
     assert rc == -1 and b"c6_forward_cascade" in lib.c6_last_error()
+
+
+def test_grouped_pack_equals_one_pack_per_model(cuda):
+    """c6_pack_weights_grouped (all checkpoints of an ensemble in two launches, from the stacked
+    tensors) writes what c6_pack_weights writes model by model, in every arithmetic mode."""
+    from pathlib import Path
+
+    from connect6_amd.model import pack_state
+
+    cfg = {"architecture_version": 4, "kernels": list(R.DEFAULT_KERNELS), "channels": list(R.DEFAULT_CHANNELS)}
+    cps = [c6.HistoricalCheckpoint(path=Path(f"m{i}.pt"), update=i + 1, model_state=R.init_state(50 + i, "torch_default"),
+                                   model_config=cfg, game_config={"board_size": 19, "win_length": 6}) for i in range(5)]
+    first = _lib.packed_bytes(_lib.PREC_BF16)
+    second_at = (first + 255) // 256 * 256
+    for name, dtype in (("fp32", torch.float32), ("bf16", torch.bfloat16), ("fp16", torch.float16),
+                        ("bf16f6", torch.bfloat16), ("bf16c", torch.bfloat16)):
+        ens = c6.HistoricalPolicyEnsemble(cps, cuda, dtype=dtype, precision=name)
+        packed = ens._packed_weights()
+        one = _lib.packed_bytes(ens._prec)
+        assert packed.shape == (5, one)
+        # bytes every mode defines: all fragments and the fp32 tail; the eight scale words behind
+        # it only where a low-order copy exists; the cascade's alignment gap not at all
+        if name == "bf16c":
+            spans = [(0, first - 32), (second_at, one)]
+        else:
+            spans = [(0, one if name == "bf16f6" else one - 32)]
+        for m in range(5):
+            alone = torch.empty(one, dtype=torch.uint8, device=cuda)
+            pack_state(ens._model_state(m), ens._prec, alone)
+            for a, b in spans:
+                assert torch.equal(packed[m, a:b], alone[a:b]), (name, m, a, b)

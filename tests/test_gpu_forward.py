@@ -456,10 +456,10 @@ def test_argmax_margin_over_32_seeds_two_inits_two_densities(cuda):
     for init in ("reference", "torch_default"):
         for st in boards:
             c, f6, plain = t[(init, st, "bf16c")], t[(init, st, "bf16f6")], t[(init, st, "bf16")]
-            # the cascade gives up next to nothing: in the mean under 0.05 %, on a single network at
-            # most 0.15 % (0.3 % on the flat-logit networks of PyTorch's default initialisation,
-            # where a quarter of the boards sit near the threshold)
-            assert bool((c >= f6 - (0.0015 if init == "reference" else 0.003)).all())
+            # the cascade gives up next to nothing: in the mean 0.01-0.02 % (bound 0.05 %), on a
+            # single network at most 0.15 % (bound 0.2 %; 0.3 % on the flat-logit networks of PyTorch's
+            # default initialisation, where a quarter of the boards sit near the threshold)
+            assert bool((c >= f6 - (0.002 if init == "reference" else 0.003)).all())
             assert c.mean() >= f6.mean() - 0.0005
             assert bool((f6 >= plain).all())               # the correction never hurts
     ref200, ref20 = t[("reference", 200, "bf16c")], t[("reference", 20, "bf16c")]
@@ -470,7 +470,7 @@ def test_argmax_margin_over_32_seeds_two_inits_two_densities(cuda):
     assert td20.mean() >= ARGMAX_MIN + 0.005 and td20.min() >= 0.96 and int((td20 < 0.99).sum()) <= 4
     assert t[("reference", 200, "bf16")].mean() < ARGMAX_MIN     # why plain bf16 is not the default
     # what the cascade costs on networks with the reference's initialisation
-    assert torch.tensor(twice[("reference", 200)]).mean() <= 0.10
+    assert torch.tensor(twice[("reference", 200)]).mean() <= 0.08
 
 
 @pytest.mark.parametrize("prec", ["bf16c", "bf16f6", "bf16", "fp16"])

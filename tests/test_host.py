@@ -97,12 +97,15 @@ def test_entry_points_reject_bad_arguments_before_touching_the_device():
     assert lib.c6_forward(None, 0, 1, 4, None, 0, _lib.PREC_BF16C, None, None, 0, None, 0.0, None, 1.0, None, None,
                           None) == -1
     assert b"c6_forward_cascade" in lib.c6_last_error()
-    assert lib.c6_forward_cascade(None, 0, 1, 4, None, 0, None, None, 0, None, 0.0, None, 1.0, None, None, 0.03,
+    assert lib.c6_forward_cascade(None, 0, 1, 4, None, 0, None, 0, None, 0, None, 0.0, None, 1.0, None, None, 0.03,
                                   None, 0, None) == -1
-    assert lib.c6_forward_cascade(None, 0, 1, 0, None, 0, None, None, 0, None, 0.0, None, 1.0, None, None, 0.03,
+    assert lib.c6_forward_cascade(None, 0, 1, 0, None, 0, None, 0, None, 0, None, 0.0, None, 1.0, None, None, 0.03,
                                   None, 0, None) == 0
-    assert lib.c6_forward_boards_cascade(None, None, None, 4, None, 0, 4, None, None, None, 1, 0.0, None, 1.0,
+    assert lib.c6_forward_cascade(None, 0, 1, 4, None, 0, None, 9, None, 0, None, 0.0, None, 1.0, None, None, 0.03,
+                                  None, 0, None) == -1                  # unknown element type of the logits
+    assert lib.c6_forward_boards_cascade(None, None, None, 4, None, 0, 4, None, None, 0, None, 1, 0.0, None, 1.0,
                                          None, None, 0.03, None, 0, None) == -1
+    assert lib.c6_pack_weights_grouped(None, None, None, None, None, None, 0, 1, None, 0, None) == -1
     size = ctypes.c_size_t(0)
     assert lib.c6_cascade_workspace_bytes(-1, ctypes.byref(size)) == -1
     assert lib.c6_cascade_workspace_bytes(4096, ctypes.byref(size)) == 0 and size.value == 16 + 4 * 4096

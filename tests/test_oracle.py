@@ -375,6 +375,9 @@ def test_cascade_rule_against_a_plain_python_loop():
     free[1] = False; free[1, 17] = True                # one free square: nothing to decide
     free[2] = False                                    # none
     logits[3, 5] = logits[3, 200] = 50.0; free[3, 5] = free[3, 200] = True   # a tie at the top
+    free[4] = False; free[4, 3] = free[4, 300] = True  # two free squares: no third to look at
+    logits[5] = 0.0; free[5] = True; logits[5, 360] = 1.0                      # a clear lead of the best ...
+    logits[5, 359] = logits[5, 358] = 1.0 - 0.0041                             # ... but two others close behind
     for thr in (0.0, 0.03, 0.5, -1.0):
         got = Q.cascade_second_pass(logits, free, thr).tolist()
         for b in range(40):
@@ -386,6 +389,8 @@ def test_cascade_rule_against_a_plain_python_loop():
             else:
                 mean = sum(z) / len(z)
                 std = math.sqrt(sum((v - mean) ** 2 for v in z) / len(z))
-                want = (z[0] - z[1]) < thr * std
+                want = (z[0] - z[1]) < thr * std or (len(z) >= 3 and (z[0] - z[2]) < 2 * thr * std)
             assert got[b] == want, (thr, b)
     assert Q.cascade_second_pass(logits, free, 0.03)[3] and not Q.cascade_second_pass(logits, free, 0.03)[0]
+    # board 5: lead 0.0041 = 0.045 standard deviations: not below 0.03, but two squares within 0.06
+    assert Q.cascade_second_pass(logits, free, 0.03)[5] and not Q.cascade_second_pass(logits, free, 0.02)[5]
