@@ -20,9 +20,10 @@ _SOURCES = ("c6_forward.hip", "c6_tail.hip", "c6_generic.hip", "c6_env.hip", "c6
 _RESOURCES = _LIBDIR / "resource_usage.txt"   # registers, scratch and LDS of every kernel, written by build()
 
 # arithmetic modes (include/connect6_amd.h)
-PREC_F32, PREC_BF16, PREC_F16, PREC_BF16F6, PREC_BF16C = 0, 1, 2, 3, 4
-PREC_BY_NAME = {"fp32": PREC_F32, "bf16": PREC_BF16, "fp16": PREC_F16, "bf16f6": PREC_BF16F6, "bf16c": PREC_BF16C}
-# cascade mode: a board is evaluated a second time (corrected arithmetic) when its best free
+PREC_F32, PREC_BF16, PREC_F16, PREC_BF16F6, PREC_BF16C, PREC_BF16F6W = 0, 1, 2, 3, 4, 5
+PREC_BY_NAME = {"fp32": PREC_F32, "bf16": PREC_BF16, "fp16": PREC_F16, "bf16f6": PREC_BF16F6, "bf16c": PREC_BF16C,
+                "bf16f6w": PREC_BF16F6W}
+# cascade mode: a board is evaluated a second time (low parts of activations and weights carried) when its best free
 # square leads the second best by less than this many standard deviations of its logits, or two
 # other free squares lie within twice that.  The plain pass's error on a difference of two logits
 # has a standard deviation of about 0.01 standard deviations of the logits: the threshold is two
@@ -45,6 +46,7 @@ EXPORTS = (
     "c6_forward_boards_cascade",
     "c6_generic_workspace_bytes",
     "c6_forward_generic",
+    "c6_forward_generic_grouped",
     "c6_forward_generic_static",
     "c6_mask_logits",
     "c6_softmax_sample",
@@ -194,6 +196,10 @@ def load() -> ctypes.CDLL:
     lib.c6_forward_generic.argtypes = [vp, i32, i64, i32, i32, ip, ip, ctypes.POINTER(vp),
                                        ctypes.POINTER(vp), vp, vp, vp, vp, i32, vp,
                                        ctypes.c_size_t, vp, vp, i32, vp, f32, vp]
+    lib.c6_forward_generic_grouped.restype = i32
+    lib.c6_forward_generic_grouped.argtypes = [vp, i32, i64, i64, i32, i32, ip, ip, ctypes.POINTER(vp),
+                                               ctypes.POINTER(vp), vp, vp, vp, vp, i32, vp,
+                                               ctypes.c_size_t, vp, vp, i32, vp, f32, vp]
     lib.c6_forward_generic_static.restype = i32
     lib.c6_forward_generic_static.argtypes = [vp, i32, i64, i32, i32, ip, ip, ctypes.POINTER(vp),
                                               ctypes.POINTER(vp), vp, vp, vp, vp, i32, vp, vp,

@@ -27,7 +27,7 @@ int launch_sample(const float *, const uint8_t *, const float *, float, long lon
 int launch_d4_expand(const void *, int, long long, void *, hipStream_t);
 int launch_d4_reduce(const float *, const float *, long long, float *, float *, hipStream_t);
 size_t generic_workspace_bytes(long long batch, int n, int layers, const int *channels);
-int launch_generic(const void *x, int x_dtype, long long batch, int n, int layers,
+int launch_generic(const void *x, int x_dtype, long long batch, long long per_group, int n, int layers,
                    const int *kernels, const int *channels, const float *const *conv_w,
                    const float *const *conv_b, const float *pol_w, const float *pol_b,
                    const float *val_w, const float *val_b, int prec, void *workspace,
@@ -78,7 +78,7 @@ static int device_ok(const char *who) {
 
 static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 static int elem_bytes(int dt) { return dt == C6_DT_F32 ? 4 : ((dt == C6_DT_BF16 || dt == C6_DT_F16) ? 2 : 0); }
-static bool valid_prec(int p) { return p >= C6_PREC_F32 && p <= C6_PREC_BF16C; }
+static bool valid_prec(int p) { return p >= C6_PREC_F32 && p <= C6_PREC_BF16F6W; }
 
 // the cascade's workspace argument, checked; `who` names the entry point in the message
 static int check_cascade_workspace(const char *who, long long boards, const void *workspace, size_t bytes) {
@@ -376,44 +376,76 @@ int c6_generic_workspace_bytes(int64_t batch, int board, int layers, const int *
   return C6_OK;
 }
 
+static int forward_generic(const char *who, const void *x, int x_dtype, int64_t groups,
+                           int64_t boards_per_group, int board, int layers, const int *kernels,
+                           const int *channels, const float *const *conv_w,
+                           const float *const *conv_b, const float *pol_w, const float *pol_b,
+                           const float *val_w, const float *val_b, int prec, void *workspace,
+                           size_t workspace_bytes, float *logits, float *value, int mask_mode,
+                           const uint8_t *legal, float fill, void *stream) {
+  if (!valid_prec(prec) || elem_bytes(x_dtype) == 0 || groups < 1 || boards_per_group < 0 ||
+      kernels == nullptr || (boards_per_group > 0 && groups > INT64_MAX / boards_per_group)) {
+    set_error("%s: bad precision %d, input type %d, groups %lld, boards %lld or null kernels", who,
+              prec, x_dtype, (long long)groups, (long long)boards_per_group);
+    return C6_EINVAL;
+  }
+  const int rc = check_arch(who, board, layers, kernels, channels);
+  if (rc != C6_OK) return rc;
+  const int64_t batch = groups * boards_per_group;
+  if (batch == 0) return C6_OK;
+  if (x == nullptr || conv_w == nullptr || pol_w == nullptr || workspace == nullptr ||
+      (value != nullptr && val_w == nullptr)) {
+    set_error("%s: null pointer (x, conv_w, pol_w, workspace, or value without val_w)", who);
+    return C6_EINVAL;
+  }
+  for (int l = 0; l < layers; ++l)
+    if (conv_w[l] == nullptr) {
+      set_error("%s: conv_w[%d] is null", who, l);
+      return C6_EINVAL;
+    }
+  if (workspace_bytes < generic_workspace_bytes(batch, board, layers, channels) ||
+      !aligned16(workspace)) {
+    set_error("%s: workspace too small or not 16-byte aligned", who);
+    return C6_EINVAL;
+  }
+  if (mask_mode < C6_MASK_NONE || mask_mode > C6_MASK_LEGAL ||
+      (mask_mode == C6_MASK_LEGAL && legal == nullptr)) {
+    set_error("%s: bad mask_mode %d", who, mask_mode);
+    return C6_EINVAL;
+  }
+  C6_REQUIRE_DEVICE(who);
+  return launch_generic(x, x_dtype, batch, boards_per_group, board, layers, kernels, channels,
+                        conv_w, conv_b, pol_w, pol_b, val_w, val_b, prec, workspace, logits, value,
+                        mask_mode, legal, fill, static_cast<hipStream_t>(stream));
+}
+
 int c6_forward_generic(const void *x, int x_dtype, int64_t batch, int board, int layers,
                        const int *kernels, const int *channels, const float *const *conv_w,
                        const float *const *conv_b, const float *pol_w, const float *pol_b,
                        const float *val_w, const float *val_b, int prec, void *workspace,
                        size_t workspace_bytes, float *logits, float *value, int mask_mode,
                        const uint8_t *legal, float fill, void *stream) {
-  if (!valid_prec(prec) || elem_bytes(x_dtype) == 0 || batch < 0 || kernels == nullptr) {
-    set_error("c6_forward_generic: bad precision %d, input type %d, batch %lld or null kernels",
-              prec, x_dtype, (long long)batch);
+  if (batch < 0) {
+    set_error("c6_forward_generic: negative batch");
     return C6_EINVAL;
   }
-  const int rc = check_arch("c6_forward_generic", board, layers, kernels, channels);
-  if (rc != C6_OK) return rc;
-  if (batch == 0) return C6_OK;
-  if (x == nullptr || conv_w == nullptr || pol_w == nullptr || workspace == nullptr ||
-      (value != nullptr && val_w == nullptr)) {
-    set_error("c6_forward_generic: null pointer (x, conv_w, pol_w, workspace, or value without val_w)");
-    return C6_EINVAL;
-  }
-  for (int l = 0; l < layers; ++l)
-    if (conv_w[l] == nullptr) {
-      set_error("c6_forward_generic: conv_w[%d] is null", l);
-      return C6_EINVAL;
-    }
-  if (workspace_bytes < generic_workspace_bytes(batch, board, layers, channels) ||
-      !aligned16(workspace)) {
-    set_error("c6_forward_generic: workspace too small or not 16-byte aligned");
-    return C6_EINVAL;
-  }
-  if (mask_mode < C6_MASK_NONE || mask_mode > C6_MASK_LEGAL ||
-      (mask_mode == C6_MASK_LEGAL && legal == nullptr)) {
-    set_error("c6_forward_generic: bad mask_mode %d", mask_mode);
-    return C6_EINVAL;
-  }
-  C6_REQUIRE_DEVICE("c6_forward_generic");
-  return launch_generic(x, x_dtype, batch, board, layers, kernels, channels, conv_w, conv_b,
-                        pol_w, pol_b, val_w, val_b, prec, workspace, logits, value, mask_mode,
-                        legal, fill, static_cast<hipStream_t>(stream));
+  return forward_generic("c6_forward_generic", x, x_dtype, 1, batch, board, layers, kernels,
+                         channels, conv_w, conv_b, pol_w, pol_b, val_w, val_b, prec, workspace,
+                         workspace_bytes, logits, value, mask_mode, legal, fill, stream);
+}
+
+int c6_forward_generic_grouped(const void *x, int x_dtype, int64_t groups,
+                               int64_t boards_per_group, int board, int layers,
+                               const int *kernels, const int *channels,
+                               const float *const *conv_w, const float *const *conv_b,
+                               const float *pol_w, const float *pol_b, const float *val_w,
+                               const float *val_b, int prec, void *workspace,
+                               size_t workspace_bytes, float *logits, float *value, int mask_mode,
+                               const uint8_t *legal, float fill, void *stream) {
+  return forward_generic("c6_forward_generic_grouped", x, x_dtype, groups, boards_per_group, board,
+                         layers, kernels, channels, conv_w, conv_b, pol_w, pol_b, val_w, val_b,
+                         prec, workspace, workspace_bytes, logits, value, mask_mode, legal, fill,
+                         stream);
 }
 
 int c6_forward_generic_static(const void *x, int x_dtype, int64_t batch, int board, int layers,

@@ -56,6 +56,7 @@ constexpr int kOverreadFrags = 8 * 3;  // zero frags after the last layer (prefe
 
 // precision policies ----------------------------------------------------------
 struct PrecF32 {
+  static constexpr int WLO = 0;
   static constexpr int PIPE = 0;      // runs the layer-by-layer kernel
   static constexpr int ID = C6_PREC_F32;
   static constexpr int EB = 4;        // bytes per element
@@ -63,6 +64,7 @@ struct PrecF32 {
   static constexpr int LO_MASK = 0;
 };
 struct PrecBF16 {
+  static constexpr int WLO = 0;
   static constexpr int PIPE = 1;      // runs the pipelined kernel (weights packed phase-major)
   static constexpr int ID = C6_PREC_BF16;
   static constexpr int EB = 2;
@@ -70,6 +72,7 @@ struct PrecBF16 {
   static constexpr int LO_MASK = 0;
 };
 struct PrecF16 {
+  static constexpr int WLO = 0;
   static constexpr int PIPE = 1;
   static constexpr int ID = C6_PREC_F16;
   static constexpr int EB = 2;
@@ -77,6 +80,7 @@ struct PrecF16 {
   static constexpr int LO_MASK = 0;
 };
 struct PrecBF16F6 {
+  static constexpr int WLO = 0;
   static constexpr int PIPE = 1;
   static constexpr int ID = C6_PREC_BF16F6;
   static constexpr int EB = 2;
@@ -91,6 +95,21 @@ struct PrecBF16F6 {
 #define C6_LO_MASK 0xfe
 #endif
   static constexpr int LO_MASK = C6_LO_MASK;
+};
+
+// bf16 + fp6 + the weights' low part: PrecBF16F6 with every weight fragment of the main pass
+// followed by a second fragment holding what the weights' rounding to bf16 dropped, itself
+// rounded to bf16 (w = hi + lo to 16 mantissa bits); each activation fragment is contracted with
+// both.  Twice the bf16 matrix work of the plain pass; what is left against fp32 arithmetic is
+// the e2m3 rounding of the activations' low part (measured 2e-4 relative L2 on the logits).  The
+// cascade's second pass.
+struct PrecBF16F6W {
+  static constexpr int WLO = 1;
+  static constexpr int PIPE = 1;
+  static constexpr int ID = C6_PREC_BF16F6W;
+  static constexpr int EB = 2;
+  static constexpr int LO6 = 1;
+  static constexpr int LO_MASK = 0xfe;
 };
 
 // bf16 + fp6 mode: what rounding an activation to bf16 drops (|lo| <= 2^-9 |a|) is contracted
@@ -117,6 +136,7 @@ template <class P> struct Geo {
   static constexpr int EB = P::EB;
   static constexpr int E = 16 / EB;                 // elements per 16-byte fragment lane
   static constexpr int KSTEP = 2 * E;               // K elements contracted per fragment pair
+  static constexpr int W = P::WLO ? 2 : 1;          // weight fragments per (k-step, cout tile): hi, or hi then lo
   static constexpr int PLANE = kChSlots * EB;       // bytes of one precision plane of a position
   static constexpr int LO_OFF = PLANE;              // the fp6 blocks follow the bf16 plane
   static constexpr int RECB = PLANE + (P::LO6 ? kChSlots : 0);  // payload bytes
@@ -148,7 +168,7 @@ template <class P> struct Geo {
   static constexpr int LDS_BYTES = P::PIPE ? NEXT_IN_OFF + (NEXT_IN_BYTES_AT + 384) * 4 : TAIL_LDS_OFF;
 
   static constexpr int layer_steps(int l) { return l == 0 ? STEPS1 : 9 * kCinArr[l] / KSTEP; }
-  static constexpr int layer_frags(int l) { return layer_steps(l) * (kCoutArr[l] / 32); }
+  static constexpr int layer_frags(int l) { return layer_steps(l) * (kCoutArr[l] / 32) * W; }
   static constexpr int frag_offset(int l) {  // in 1 KiB fragments
     int s = 0;
     for (int i = 0; i < l; ++i) s += layer_frags(i);
@@ -179,9 +199,10 @@ template <class P> struct Geo {
   // lane's square), one coalesced 16-byte load per lane each.
   static constexpr int FAST1_STEPS = kK1 * CPR;
   static constexpr int FAST1_OFF = HI_FRAGS + LO_FRAGS;  // in 1 KiB fragments
-  static constexpr int PLANE2_FRAG_OFF = FAST1_OFF + FAST1_STEPS + 8;  // (8 zero fragments: over-read)
+  static constexpr int FAST1_STREAM = FAST1_STEPS * W;   // fragments of that copy
+  static constexpr int PLANE2_FRAG_OFF = FAST1_OFF + FAST1_STREAM + 8;  // (8 zero fragments: over-read)
   static constexpr int PLANE2_FRAGS = kWaves * 3 * 4;
-  static constexpr int FAST1_FRAGS = (P::PIPE && EB == 2) ? FAST1_STEPS + 8 + PLANE2_FRAGS : 0;
+  static constexpr int FAST1_FRAGS = (P::PIPE && EB == 2) ? FAST1_STREAM + 8 + PLANE2_FRAGS : 0;
   static constexpr int TOTAL_FRAGS = HI_FRAGS + LO_FRAGS + FAST1_FRAGS;
   static constexpr size_t TAIL_OFF = (size_t)TOTAL_FRAGS * 1024;  // fp32 tail: biases, heads
   // tail words: bias[544] polw[96] valw[96] polb valb pad pad, then 8 ints sw[layer]
@@ -191,9 +212,10 @@ template <class P> struct Geo {
 };
 
 // Cascade mode (C6_PREC_BF16C): one packed set = the plain bf16 set, then (256-byte aligned)
-// the bf16 + fp6 set of the same parameters.
+// the set of the same parameters for the second pass (bf16 + fp6 + the weights' low part).
+using PrecCascadeSecond = PrecBF16F6W;
 constexpr size_t kCascadeSecondOffset = (Geo<PrecBF16>::PACKED_BYTES + 255) & ~(size_t)255;
-constexpr size_t kCascadePackedBytes = kCascadeSecondOffset + Geo<PrecBF16F6>::PACKED_BYTES;
+constexpr size_t kCascadePackedBytes = kCascadeSecondOffset + Geo<PrecCascadeSecond>::PACKED_BYTES;
 // its workspace: int32 count (+ 3 words of padding), then one int32 per board
 constexpr size_t cascade_workspace_bytes(long long boards) { return (size_t)(16 + 4 * boards + 15) & ~(size_t)15; }
 

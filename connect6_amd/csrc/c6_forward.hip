@@ -45,6 +45,9 @@ template <> __device__ __forceinline__ void mma<PrecBF16>(const v4i &a, const v4
 template <> __device__ __forceinline__ void mma<PrecBF16F6>(const v4i &a, const v4i &b, f32x16 &c) {
   mma<PrecBF16>(a, b, c);
 }
+template <> __device__ __forceinline__ void mma<PrecBF16F6W>(const v4i &a, const v4i &b, f32x16 &c) {
+  mma<PrecBF16>(a, b, c);
+}
 template <> __device__ __forceinline__ void mma<PrecF16>(const v4i &a, const v4i &b, f32x16 &c) {
   c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
                                              __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
@@ -253,8 +256,9 @@ __device__ __forceinline__ void conv1_pass(const unsigned char *smem, const WFra
                                            f32x16 (&acc)[1][3]) {
   using G = Geo<P>;
   using PP = L1Pipe<P>;
-  constexpr int CPR = PP::CPR, U = PP::U, D = PP::D, ITERS = PP::ITERS;
+  constexpr int CPR = PP::CPR, U = PP::U, D = PP::D, ITERS = PP::ITERS, W = G::W;
   constexpr int ROWB = kL1RowPitch * G::EB;
+  static_assert((U * W) % D == 0, "the ring must line up across loop iterations");
 
   // activation fragments are fetched kAhead k-steps before their MFMAs (an LDS read issued
   // during one k-step of three MFMAs would not be back by the next)
@@ -268,7 +272,7 @@ __device__ __forceinline__ void conv1_pass(const unsigned char *smem, const WFra
 #pragma unroll 1
   for (int it = 0; it < ITERS; ++it) {
     const int adv = it * PP::ROWS_BODY * ROWB;
-    const WFrags wn = wl + (it * U + D);
+    const WFrags wn = wl + (it * U * W + D);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       // after the last steps this reads the zero row / the next copy, which is harmless
@@ -278,9 +282,12 @@ __device__ __forceinline__ void conv1_pass(const unsigned char *smem, const WFra
       for (int j = 0; j < 3; ++j)
         bq[un % (kAhead + 1)][j] = *reinterpret_cast<const v4i *>(smem + l1base[j] + adv + offn);
 #pragma unroll
-      for (int j = 0; j < 3; ++j) mma<P>(ring[u % D][0], bq[u % (kAhead + 1)][j], acc[0][j]);
-      ring[u % D][0] = wn[u];  // k-step it*U + u + D (the tail over-reads the next layer)
-      interleave_step<3 * (P::EB == 4 ? 4 : 1), 3, 1>();
+      for (int w = 0; w < W; ++w) {  // the weights, then (WLO) what their rounding dropped
+#pragma unroll
+        for (int j = 0; j < 3; ++j) mma<P>(ring[(u * W + w) % D][0], bq[u % (kAhead + 1)][j], acc[0][j]);
+        ring[(u * W + w) % D][0] = wn[u * W + w];  // fragment (it*U + u) * W + w + D (the tail over-reads the next layer)
+      }
+      interleave_step<3 * W * (P::EB == 4 ? 4 : 1), 3, W>();
       __builtin_amdgcn_sched_barrier(0);
     }
   }
@@ -294,7 +301,7 @@ __device__ __forceinline__ void conv1_fast_pass(const unsigned char *smem, const
                                                 v4i (&ring)[L1Pipe<P>::D][1], const int (&l1fast)[3],
                                                 f32x16 (&acc)[1][3]) {
   using G = Geo<P>;
-  constexpr int CPR = G::CPR, D = L1Pipe<P>::D, QN = kAhead + 1, S = G::FAST1_STEPS;
+  constexpr int CPR = G::CPR, D = L1Pipe<P>::D, QN = kAhead + 1, S = G::FAST1_STEPS, W = G::W;
   constexpr int ROWB = kL1RowPitch * G::EB;
   static_assert(S % QN == 0, "fragment queue must line up");
   auto frag = [&](int j, int s) {  // kernel row s / CPR is three halo rows further down
@@ -312,9 +319,13 @@ __device__ __forceinline__ void conv1_fast_pass(const unsigned char *smem, const
       for (int j = 0; j < 3; ++j) bq[(s + kAhead) % QN][j] = frag(j, s + kAhead);
     }
 #pragma unroll
-    for (int j = 0; j < 3; ++j) mma<P>(ring[s % D][0], bq[s % QN][j], acc[0][j]);
-    ring[s % D][0] = wl[s + D];  // (the tail over-reads the zero fragments behind the stream)
-    interleave_step<3, 3, 1>();
+    for (int w = 0; w < W; ++w) {
+      constexpr int f0 = s * W;
+#pragma unroll
+      for (int j = 0; j < 3; ++j) mma<P>(ring[(f0 + w) % D][0], bq[s % QN][j], acc[0][j]);
+      ring[(f0 + w) % D][0] = wl[f0 + w + D];  // (the tail over-reads the zero fragments behind the stream)
+    }
+    interleave_step<3 * W, 3, W>();
     __builtin_amdgcn_sched_barrier(0);
   });
 }
@@ -967,14 +978,18 @@ __device__ __forceinline__ void conv3_seg(const unsigned char *smem, const WFrag
                                           const int (&rb)[3], f32x16 (&acc)[kCoutArr[L] / 32][3],
                                           const f32x16 (&bias)[kCoutArr[L] / 32], Hidden hidden) {
   using G = Geo<P>;
-  constexpr int NT = kCoutArr[L] / 32, NTP = kCinArr[L] / 32;
+  constexpr int NT = kCoutArr[L] / 32, NTP = kCinArr[L] / 32, W = G::W;
   constexpr int U = kPhaseSteps, RN = kRing * NT, QN = kAhead + 1;
   constexpr int T0 = KIND == kSegB ? 1 : 0;
   constexpr int NTS = KIND == kSegFull ? NT : (KIND == kSegA ? 1 : NT - 1);
-  constexpr int F0 = PH * U * NT + (KIND == kSegB ? U : 0);
+  // (WLO: every weight fragment is followed by the fragment of what its rounding dropped; the two
+  // meet the same activation fragment and the same accumulator, so a tile takes W MFMAs per
+  // k-step and pixel tile, and the ring, unchanged in size, reaches kRing / W k-steps ahead)
+  constexpr int NV = NTS * W;
+  constexpr int F0 = (PH * U * NT + (KIND == kSegB ? U : 0)) * W;
   constexpr int KS0 = KIND == kSegB ? U : 0;
   constexpr int BLK = (act_rot(L) + PH) % 3;
-  static_assert(G::KSTEP == 16 && G::PADDED && U % QN == 0 && (U * NTP * NT) % RN == 0, "segment shape");
+  static_assert(G::KSTEP == 16 && G::PADDED && U % QN == 0 && (U * NTP * NT * W) % RN == 0, "segment shape");
   static_assert(KIND == kSegFull || (PH == NTP - 1 && NT > 1), "parts A and B split the last phase");
   auto frag = [&](int j, int u) {
     const int tap = u / 2;
@@ -987,13 +1002,13 @@ __device__ __forceinline__ void conv3_seg(const unsigned char *smem, const WFrag
 #pragma unroll
       for (int j = 0; j < 3; ++j) bq[a][j] = frag(j, a);
   }
-  static_for<0, U * NTS * 3>([&](auto gc) __attribute__((always_inline)) {
+  static_for<0, U * NV * 3>([&](auto gc) __attribute__((always_inline)) {
     constexpr int g = decltype(gc)::value;
-    constexpr int u = g / (NTS * 3), ti = (g / 3) % NTS, t = T0 + ti, j = g % 3;
-    constexpr int f = F0 + u * NTS + ti;
+    constexpr int u = g / (NV * 3), vi = (g / 3) % NV, ti = vi / W, t = T0 + ti, j = g % 3;
+    constexpr int f = F0 + u * NV + vi;
     // (a layer with one input tile runs its low-order pass first, and that one starts from the bias)
     constexpr bool kLoFirst = P::LO6 && ((P::LO_MASK >> L) & 1) && NTP == 1;
-    if constexpr (PH == 0 && u == 0 && !kLoFirst) {
+    if constexpr (PH == 0 && u == 0 && vi % W == 0 && !kLoFirst) {
       f32x16 c0 = bias[t];
       mma<P>(ring[f % RN], bq[(KS0 + u) % QN][j], c0);
       acc[t][j] = c0;
@@ -1001,7 +1016,7 @@ __device__ __forceinline__ void conv3_seg(const unsigned char *smem, const WFrag
       mma<P>(ring[f % RN], bq[(KS0 + u) % QN][j], acc[t][j]);
     }
     // fragments of k-step u + kAhead; part A runs on into part B, which reads the same ones again
-    if constexpr (ti == 0 && (u + kAhead < U || KIND == kSegA))
+    if constexpr (vi == 0 && (u + kAhead < U || KIND == kSegA))
       bq[(KS0 + u + kAhead) % QN][j] = frag(j, (u + kAhead) % U);
     if constexpr (j == 2) ring[f % RN] = wl[f + RN];
     hidden(g);
@@ -1065,7 +1080,7 @@ __device__ __forceinline__ void pipe_layer(
   // phases 0 .. NTP-2 carry tiles 1 .. NTP-1 of layer L-1
   static_for<0, NTP - 1>([&](auto pc) __attribute__((always_inline)) {
     constexpr int p = decltype(pc)::value;
-    using Plan = EpiPlan<P, Whole, kLoPass, true, kPhaseSteps * NT * 3 - 8>;
+    using Plan = EpiPlan<P, Whole, kLoPass, true, kPhaseSteps * NT * G::W * 3 - 8>;
     conv3_seg<P, L, kSegFull, p>(smem, wl, ring, bq, rb, acc, bias, [&](int g) __attribute__((always_inline)) {
       Plan::template run<NTP>(smem, wb, h4, prev, p + 1, (RIN + p + 1) % 3, g, carry, k);
     });
@@ -1086,7 +1101,7 @@ __device__ __forceinline__ void pipe_layer(
     conv3_seg<P, L, kSegFull, NTP - 1>(smem, wl, ring, bq, rb, acc, bias, [](int) {});
   } else {
     conv3_seg<P, L, kSegA, NTP - 1>(smem, wl, ring, bq, rb, acc, bias, [](int) {});
-    using Plan = EpiPlan<P, Whole, kLoNext, true, kPhaseSteps * (NT - 1) * 3 - 8>;
+    using Plan = EpiPlan<P, Whole, kLoNext, true, kPhaseSteps * (NT - 1) * G::W * 3 - 8>;
     conv3_seg<P, L, kSegB, NTP - 1>(smem, wl, ring, bq, rb, acc, bias, [&](int g) __attribute__((always_inline)) {
       if constexpr (!kLast) {
         Plan::template run<NT>(smem, wb, h4, acc, 0, ROUT, g, carry, k);
@@ -1856,6 +1871,18 @@ template <class P> __device__ __forceinline__ void put_elem(unsigned char *dst, 
   }
 }
 
+// part 0: the weight itself (put_elem rounds it to the storage type); part 1 (WLO): what that
+// rounding drops, which put_elem rounds in turn
+template <class P> __device__ __forceinline__ float weight_part(float v, int part) {
+  if constexpr (P::EB == 4) {
+    return v;
+  } else {
+    const float hi = __builtin_bit_cast(float, (unsigned)bits16<P>(v) << 16);
+    static_assert(P::WLO == 0 || P::ID != C6_PREC_F16, "the low part is defined for bf16 storage");
+    return part ? v - hi : v;
+  }
+}
+
 // The parameters of weight set `g` of a (possibly stacked) PackParams.
 struct GroupView {
   const PackParams &p;
@@ -1916,13 +1943,14 @@ template <class P> __global__ void pack_kernel(const PackParams all) {
         *reinterpret_cast<f32x4 *>(dst) = t4;
         return;
       }
-      if (G::FAST1_FRAGS > 0 && frag >= G::FAST1_OFF && frag < G::FAST1_OFF + G::FAST1_STEPS) {
+      if (G::FAST1_FRAGS > 0 && frag >= G::FAST1_OFF && frag < G::FAST1_OFF + G::FAST1_STREAM) {
         // k-step (ky, 8 columns); lane half = input plane
-        const int fi = frag - G::FAST1_OFF, ky = fi / G::CPR, jj = fi % G::CPR;
+        const int part = (frag - G::FAST1_OFF) % G::W;
+        const int fi = (frag - G::FAST1_OFF) / G::W, ky = fi / G::CPR, jj = fi % G::CPR;
         const float *w = prm.conv_w(0);
         for (int e = 0; e < G::E; ++e) {
           const int kx = jj * G::E + e;
-          put_elem<P>(dst, e, kx < kK1 ? w[((m * 3 + h) * kK1 + ky) * kK1 + kx] * act_scale<P>() : 0.0f);
+          put_elem<P>(dst, e, weight_part<P>(kx < kK1 ? w[((m * 3 + h) * kK1 + ky) * kK1 + kx] * act_scale<P>() : 0.0f, part));
         }
         return;
       }
@@ -1968,7 +1996,10 @@ template <class P> __global__ void pack_kernel(const PackParams all) {
       *reinterpret_cast<v4i *>(dst) = o;
       return;
     }
-    const int fi = frag - G::frag_offset(l);
+    // (WLO: fragment 2i holds the weights of fragment i of the plain order, fragment 2i + 1 what
+    // their rounding dropped)
+    const int part = (frag - G::frag_offset(l)) % G::W;
+    const int fi = (frag - G::frag_offset(l)) / G::W;
     const int cin = kCinArr[l], cout = kCoutArr[l];
     const int nt = cout / 32;
     const int s = fi / nt, t = fi - s * nt;
@@ -1982,7 +2013,7 @@ template <class P> __global__ void pack_kernel(const PackParams all) {
         const int kx = jj * G::E + e;
         float v = 0.0f;
         if (row < kK1 * 3 && kx < kK1) v = w[((co * 3 + ch) * kK1 + ky) * kK1 + kx] * act_scale<P>();
-        put_elem<P>(dst, e, v);
+        put_elem<P>(dst, e, weight_part<P>(v, part));
       }
     } else {
       // k-step s -> (tap, 16 or 8 input channels): tap-major, or for the pipelined kernel
@@ -2003,7 +2034,7 @@ template <class P> __global__ void pack_kernel(const PackParams all) {
       const int cot = 32 * tile + m;
       for (int e = 0; e < G::E; ++e) {
         const int c = cbase + h * G::E + e;
-        put_elem<P>(dst, e, w[(cot * cin + c) * 9 + tap]);
+        put_elem<P>(dst, e, weight_part<P>(w[(cot * cin + c) * 9 + tap], part));
       }
     }
     return;
@@ -2126,13 +2157,14 @@ int dispatch_pack(int prec, const PackParams &pp, hipStream_t st) {
     if (rc != C6_OK) return rc;
     PackParams second = pp;
     second.packed = pp.packed + kCascadeSecondOffset;
-    return launch_pack<PrecBF16F6>(second, st);
+    return launch_pack<PrecCascadeSecond>(second, st);
   }
   switch (prec) {
     case C6_PREC_F32: return launch_pack<PrecF32>(pp, st);
     case C6_PREC_BF16: return launch_pack<PrecBF16>(pp, st);
     case C6_PREC_F16: return launch_pack<PrecF16>(pp, st);
     case C6_PREC_BF16F6: return launch_pack<PrecBF16F6>(pp, st);
+    case C6_PREC_BF16F6W: return launch_pack<PrecBF16F6W>(pp, st);
   }
   set_error("unknown precision mode %d", prec);
   return C6_EINVAL;
@@ -2144,6 +2176,7 @@ int dispatch_forward(int prec, const FwdParams &fp, hipStream_t st) {
     case C6_PREC_BF16: return launch_forward<PrecBF16>(fp, st);
     case C6_PREC_F16: return launch_forward<PrecF16>(fp, st);
     case C6_PREC_BF16F6: return launch_forward<PrecBF16F6>(fp, st);
+    case C6_PREC_BF16F6W: return launch_forward<PrecBF16F6W>(fp, st);
   }
   set_error("unknown precision mode %d", prec);
   return C6_EINVAL;
@@ -2154,8 +2187,8 @@ __global__ void cascade_reset_kernel(int *count) {
 }
 
 // Cascade: every board through the plain bf16 kernel, which lists the boards whose decision
-// margin is below `threshold`; then the listed boards through the bf16 + fp6 kernel, which
-// overwrites their outputs.  Three launches on the caller's stream, no host synchronisation:
+// margin is below `threshold`; then the listed boards through the kernel that also carries the
+// low parts of activations and weights, which overwrites their outputs.  Three launches on the caller's stream, no host synchronisation:
 // the second kernel reads the length of the list from device memory.
 int dispatch_cascade(const FwdParams &fp, float threshold, void *workspace, hipStream_t st) {
   int *count = static_cast<int *>(workspace);
@@ -2172,7 +2205,7 @@ int dispatch_cascade(const FwdParams &fp, float threshold, void *workspace, hipS
   second.redo_mode = kRedoConsume;
   second.redo_count = count;
   second.redo_list = count + 4;
-  return launch_forward<PrecBF16F6>(second, st);
+  return launch_forward<PrecCascadeSecond>(second, st);
 }
 
 size_t packed_bytes(int prec) {
@@ -2182,6 +2215,7 @@ size_t packed_bytes(int prec) {
     case C6_PREC_BF16: return Geo<PrecBF16>::PACKED_BYTES;
     case C6_PREC_F16: return Geo<PrecF16>::PACKED_BYTES;
     case C6_PREC_BF16F6: return Geo<PrecBF16F6>::PACKED_BYTES;
+    case C6_PREC_BF16F6W: return Geo<PrecBF16F6W>::PACKED_BYTES;
   }
   return 0;
 }

@@ -57,12 +57,16 @@ __device__ __forceinline__ float load_any(const void *x, int dt, size_t i) {
   return (float)__builtin_bit_cast(_Float16, b);
 }
 
-// out[b,co,r,c] = act(bias[co] + sum_{ci,ky,kx} w[co,ci,ky,kx] * in[b,ci,r+ky-k/2,c+kx-k/2])
+// out[b,co,r,c] = act(bias[g,co] + sum_{ci,ky,kx} w[g,co,ci,ky,kx] * in[b,ci,r+ky-k/2,c+kx-k/2])
+// with g = b / per_group: the weight sets of a group of models lie one after the other
+// (connect6/history.py:224-240 stacks them that way) and board b belongs to set g -- one launch
+// per layer for the whole ensemble, as the reference's grouped convolution
+// (connect6/history.py:263-273).  A single model is per_group = batch.
 __global__ void generic_conv_kernel(const void *__restrict__ in, int in_dtype,
                                     const float *__restrict__ w, const float *__restrict__ bias,
-                                    float *__restrict__ out, long long batch, int cin, int cout,
-                                    int n, int k, int silu, int round_w, int round_a,
-                                    int round_out) {
+                                    float *__restrict__ out, long long batch, long long per_group,
+                                    int cin, int cout, int n, int k, int silu, int round_w,
+                                    int round_a, int round_out) {
   const long long total = batch * cout * n * n;
   const long long stride = (long long)gridDim.x * blockDim.x;
   const int pad = k / 2;
@@ -71,10 +75,11 @@ __global__ void generic_conv_kernel(const void *__restrict__ in, int in_dtype,
     const int r = (int)((i / n) % n);
     const int co = (int)((i / ((long long)n * n)) % cout);
     const long long b = i / ((long long)n * n * cout);
-    float acc = bias ? bias[co] : 0.0f;
+    const size_t g = (size_t)(b / per_group);
+    float acc = bias ? bias[g * cout + co] : 0.0f;
     for (int ci = 0; ci < cin; ++ci) {
       const size_t plane = ((size_t)b * cin + ci) * n * n;
-      const float *wk = w + ((size_t)co * cin + ci) * k * k;
+      const float *wk = w + ((g * cout + co) * cin + ci) * k * k;
       for (int ky = 0; ky < k; ++ky) {
         const int rr = r + ky - pad;
         if (rr < 0 || rr >= n) continue;
@@ -97,13 +102,16 @@ __global__ __launch_bounds__(256) void generic_heads_kernel(
     const float *__restrict__ pol_b, const float *__restrict__ val_w,
     const float *__restrict__ val_b, const void *__restrict__ x, int x_dtype, int in_channels,
     int mask_mode, const uint8_t *__restrict__ legal, float fill, float *__restrict__ logits,
-    float *__restrict__ value) {
+    float *__restrict__ value, long long per_group) {
   __shared__ float red[256];
   const long long b = blockIdx.x;
+  const size_t g = (size_t)(b / per_group);
+  pol_w += g * channels;
+  if (val_w) val_w += g * channels;
   const int nn = n * n;
   float vsum = 0.0f;
   for (int p = threadIdx.x; p < nn; p += blockDim.x) {
-    float pol = pol_b ? pol_b[0] : 0.0f;
+    float pol = pol_b ? pol_b[g] : 0.0f;
     float val = 0.0f;
     for (int c = 0; c < channels; ++c) {
       const float f = feat[((size_t)b * channels + c) * nn + p];
@@ -127,7 +135,7 @@ __global__ __launch_bounds__(256) void generic_heads_kernel(
     __syncthreads();
   }
   if (threadIdx.x == 0 && value != nullptr)
-    value[b] = tanhf(red[0] / (float)nn + (val_b ? val_b[0] : 0.0f));
+    value[b] = tanhf(red[0] / (float)nn + (val_b ? val_b[g] : 0.0f));
 }
 
 static unsigned blocks_for(long long items) {
@@ -142,8 +150,8 @@ size_t generic_workspace_bytes(long long batch, int n, int layers, const int *ch
   return 2 * (size_t)batch * cmax * n * n * sizeof(float);
 }
 
-int launch_generic(const void *x, int x_dtype, long long batch, int n, int layers,
-                   const int *kernels, const int *channels, const float *const *conv_w,
+int launch_generic(const void *x, int x_dtype, long long batch, long long per_group, int n,
+                   int layers, const int *kernels, const int *channels, const float *const *conv_w,
                    const float *const *conv_b, const float *pol_w, const float *pol_b,
                    const float *val_w, const float *val_b, int prec, void *workspace,
                    float *logits, float *value, int mask_mode, const uint8_t *legal, float fill,
@@ -153,7 +161,10 @@ int launch_generic(const void *x, int x_dtype, long long batch, int n, int layer
   float *buf[2] = {static_cast<float *>(workspace),
                    static_cast<float *>(workspace) + (size_t)batch * cmax * n * n};
   // arithmetic contract of each mode: which operands are rounded to 16 bits
-  const int round_w = prec == C6_PREC_F32 ? C6_DT_F32 : (prec == C6_PREC_F16 ? C6_DT_F16 : C6_DT_BF16);
+  // (C6_PREC_BF16F6W carries the weights' low part as well: nothing is rounded)
+  const int round_w = (prec == C6_PREC_F32 || prec == C6_PREC_BF16F6W)
+                          ? C6_DT_F32
+                          : (prec == C6_PREC_F16 ? C6_DT_F16 : C6_DT_BF16);
   // (the hi+lo modes carry the activations' low-order bits: no activation rounding here)
   const int round_a = prec == C6_PREC_BF16 ? C6_DT_BF16 : (prec == C6_PREC_F16 ? C6_DT_F16 : C6_DT_F32);
   const void *in = x;
@@ -164,7 +175,8 @@ int launch_generic(const void *x, int x_dtype, long long batch, int n, int layer
     const int last = l + 1 == layers;
     hipLaunchKernelGGL(generic_conv_kernel, dim3(blocks_for(batch * channels[l] * n * n)),
                        dim3(256), 0, st, in, in_dtype, conv_w[l], conv_b ? conv_b[l] : nullptr,
-                       out, batch, cin, channels[l], n, kernels[l], 1, round_w, round_a,
+                       out, batch, per_group, cin, channels[l], n, kernels[l], 1, round_w,
+                       round_a,
                        last ? C6_DT_F32 : round_a);
     in = out;
     in_dtype = C6_DT_F32;
@@ -172,7 +184,7 @@ int launch_generic(const void *x, int x_dtype, long long batch, int n, int layer
   }
   hipLaunchKernelGGL(generic_heads_kernel, dim3((unsigned)batch), dim3(256), 0, st,
                      static_cast<const float *>(in), cin, n, pol_w, pol_b, val_w, val_b, x,
-                     x_dtype, 3, mask_mode, legal, fill, logits, value);
+                     x_dtype, 3, mask_mode, legal, fill, logits, value, per_group);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) {
     set_error("generic forward launch failed: %s", hipGetErrorString(e));

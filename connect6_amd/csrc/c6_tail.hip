@@ -64,7 +64,7 @@ __global__ void mask_elem_kernel(const T *__restrict__ in, const uint8_t *__rest
 
 // Rows of 361 elements are only 4-byte aligned, but FOUR consecutive rows span 4*361*4 =
 // 16*361 bytes and start 16-byte aligned (the tensor base is).  The kernels below therefore
-// work on groups of four boards (eight planes for the view gather) and move them with 16-byte
+// work on groups of four boards (32 planes for the view gather) and move them with 16-byte
 // accesses; the last, partial group falls back to element accesses.
 
 // Eight boards per group (two per wave): masked softmax over 361 logits and inverse-CDF draw
@@ -157,15 +157,21 @@ __global__ __launch_bounds__(256) void sample_kernel(const float *__restrict__ l
 }
 
 // out[p,plane,v] = x[plane, from_view(v,p)]   (connect6/train.py:222-230)
-// Each workgroup stages eight planes in LDS once and writes all eight permuted views of them:
-// the input is read once, every output element is one LDS gather, stores are 16 bytes.
-constexpr int kExpandPlanes = 8;
+// Each workgroup stages 32 planes in LDS once and writes all eight permuted views of them, one
+// view after the other: the input is read once, every output element is one LDS gather, stores
+// are 16 bytes, and a workgroup's share of a view is one contiguous run of 46,208 bytes (4-byte
+// elements) = 361 whole 128-byte lines.  The run length is what the store side is sensitive to:
+// with 8 planes per workgroup (11.5 KB runs) the same stores alone, with nothing read, take
+// 13 % longer.
+constexpr int kExpandPlanes = 32;
+constexpr int kExpandThreads = 512;
 template <typename T>
-__global__ __launch_bounds__(256) void d4_expand_kernel(const T *__restrict__ x, long long planes,
-                                                        T *__restrict__ out) {
+__global__ __launch_bounds__(kExpandThreads) void d4_expand_kernel(const T *__restrict__ x,
+                                                                   long long planes,
+                                                                   T *__restrict__ out) {
   constexpr int VEC = 16 / sizeof(T);                       // elements per 16-byte access
-  constexpr int SPAN = kExpandPlanes * kPix;                // 2888 elements: a multiple of VEC
-  static_assert(SPAN % VEC == 0, "eight planes must be whole 16-byte units");
+  constexpr int SPAN = kExpandPlanes * kPix;                // 11552 elements: a multiple of VEC
+  static_assert(SPAN % VEC == 0, "a group of planes must be whole 16-byte units");
   typedef T vec_t __attribute__((ext_vector_type(VEC)));
   __shared__ __attribute__((aligned(16))) T s_in[SPAN];
   const long long plane0 = (long long)blockIdx.x * kExpandPlanes;
@@ -177,31 +183,28 @@ __global__ __launch_bounds__(256) void d4_expand_kernel(const T *__restrict__ x,
                        ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst0) |
                          (view_stride * sizeof(T))) & 15u) == 0;
   if (aligned) {
-    for (int i = threadIdx.x; i < SPAN / VEC; i += blockDim.x)
+    for (int i = threadIdx.x; i < SPAN / VEC; i += kExpandThreads)
       reinterpret_cast<vec_t *>(s_in)[i] = reinterpret_cast<const vec_t *>(src)[i];
   } else {
-    for (int i = threadIdx.x; i < np * kPix; i += blockDim.x) s_in[i] = src[i];
+    for (int i = threadIdx.x; i < np * kPix; i += kExpandThreads) s_in[i] = src[i];
   }
   __syncthreads();
   if (aligned) {
-    for (int i = threadIdx.x; i < SPAN / VEC; i += blockDim.x) {
-      int pl[VEC], v[VEC];
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) {
-        const int idx = i * VEC + e;
-        pl[e] = idx / kPix;
-        v[e] = idx - pl[e] * kPix;
-      }
-#pragma unroll
-      for (int p = 0; p < 8; ++p) {
+    for (int p = 0; p < 8; ++p) {
+      for (int i = threadIdx.x; i < SPAN / VEC; i += kExpandThreads) {
         vec_t o;
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) o[e] = s_in[pl[e] * kPix + d4_from_view(v[e], p)];
+        for (int e = 0; e < VEC; ++e) {
+          const int idx = i * VEC + e;
+          const int pl = idx / kPix, v = idx - pl * kPix;
+          o[e] = s_in[pl * kPix + d4_from_view(v, p)];
+        }
         reinterpret_cast<vec_t *>(dst0 + p * view_stride)[i] = o;
       }
     }
   } else {
-    for (int i = threadIdx.x; i < np * kPix; i += blockDim.x) {
+    for (int i = threadIdx.x; i < np * kPix; i += kExpandThreads) {
       const int pl = i / kPix, v = i - pl * kPix;
 #pragma unroll
       for (int p = 0; p < 8; ++p) dst0[p * view_stride + i] = s_in[pl * kPix + d4_from_view(v, p)];
@@ -334,11 +337,11 @@ int launch_d4_expand(const void *x, int elem_bytes, long long batch, void *out, 
   const long long planes = batch * 3;
   const dim3 grid((unsigned)((planes + kExpandPlanes - 1) / kExpandPlanes));
   if (elem_bytes == 4)
-    hipLaunchKernelGGL(d4_expand_kernel<uint32_t>, grid, dim3(256), 0, st, (const uint32_t *)x,
-                       planes, (uint32_t *)out);
+    hipLaunchKernelGGL(d4_expand_kernel<uint32_t>, grid, dim3(kExpandThreads), 0, st,
+                       (const uint32_t *)x, planes, (uint32_t *)out);
   else
-    hipLaunchKernelGGL(d4_expand_kernel<uint16_t>, grid, dim3(256), 0, st, (const uint16_t *)x,
-                       planes, (uint16_t *)out);
+    hipLaunchKernelGGL(d4_expand_kernel<uint16_t>, grid, dim3(kExpandThreads), 0, st,
+                       (const uint16_t *)x, planes, (uint16_t *)out);
   return check_launch("d4_expand");
 }
 

@@ -36,10 +36,9 @@ def _normalized_model_cfg(cfg: dict[str, Any]) -> dict[str, Any]:
 
 
 # bfloat16 selects the cascade (plain bf16 layer boundaries, then the boards whose decision is
-# close again with the fp6 pass on what the activations' rounding dropped), the fastest bf16 mode
-# that keeps the corrected arithmetic's agreement with the fp32 argmax; the literal "round every
-# activation to bf16" arithmetic stays available as precision="bf16", the correction on every
-# board as precision="bf16f6".
+# close again with the low parts of activations and weights carried), the fastest bf16 mode that
+# keeps the argmax of fp32; the literal "round everything to bf16" arithmetic stays available as
+# precision="bf16", the corrections on every board as precision="bf16f6" / "bf16f6w".
 _PREC_OF_DTYPE = {
     torch.float32: _lib.PREC_F32,
     torch.bfloat16: _lib.PREC_BF16C,
@@ -118,6 +117,7 @@ class HistoricalPolicyEnsemble:
         self._packed: tuple | None = None   # (buffer, stream it was packed on, event)
         self._states = states
         self._stacked: dict[str, torch.Tensor | None] = {}
+        self._stacked32: dict[str, torch.Tensor] | None = None
 
     # -- the reference's stacked attributes, on `device` in `dtype`, built when first read --
     def _stacked_attr(self, key: str, optional: bool) -> torch.Tensor | None:
@@ -214,11 +214,14 @@ class HistoricalPolicyEnsemble:
             logits, _, _, _ = run_forward(x.reshape(m * t, *expected_tail), self._packed_weights(),
                                           self._prec, m, t, want_value=False,
                                           logits_dtype=self.dtype if direct else torch.float32)
-        else:  # other architectures: layer by layer, one model after the other
-            logits = torch.cat([
-                run_forward_generic(x[i], self._model_state(i), self.kernels, self.channels,
-                                    self._prec, want_value=False)[0]
-                for i in range(m)
-            ])
+        else:  # other architectures: layer by layer, every layer one launch for all models
+            keys = [f"convs.{i}.{kind}" for i in range(len(self.kernels)) for kind in ("weight", "bias")]
+            keys += ["policy_output.weight", "policy_output.bias"]
+            if self._stacked32 is None:   # the layer-by-layer kernels read fp32 parameters
+                self._stacked32 = {k: v.float().contiguous() for k in keys
+                                   if (v := self._stacked_attr(k, optional=k.endswith("bias"))) is not None}
+            stacked = self._stacked32
+            logits = run_forward_generic(x.reshape(m * t, *expected_tail), stacked, self.kernels, self.channels,
+                                         self._prec, want_value=False, groups=m)[0]
         logits = logits.view(m, t, self.action_size)
         return logits if self.dtype == torch.float32 else logits.to(self.dtype)

@@ -167,9 +167,15 @@ def run_forward_generic(
     fill: float = _FILL_LOWEST,
     static_workspace: bool = False,
     out: tuple[torch.Tensor, torch.Tensor | None] | None = None,
+    groups: int = 1,
 ):
     """Launch ``c6_forward_generic`` for one weight set of any architecture:
     x ``[B,3,n,n]`` -> (logits ``[B,n*n]``, value ``[B]`` or None).
+
+    ``groups = G > 1``: ``state`` holds G weight sets stacked along a leading dimension (as
+    ``HistoricalPolicyEnsemble._stack`` lays them out, connect6/history.py:224-240), x is
+    ``[G*T,3,n,n]`` and board b uses set ``b // T`` -- ``c6_forward_generic_grouped``, one launch
+    per layer for all sets.
 
     ``static_workspace`` routes the layer-boundary activations through the
     library's built-in 16 MiB array (``c6_forward_generic_static``) instead of
@@ -181,6 +187,8 @@ def run_forward_generic(
     b, n = int(x.shape[0]), int(x.shape[-1])
     layers = len(kernels)
     keep = []
+    if groups < 1 or b % groups or (groups > 1 and static_workspace):
+        raise ValueError(f"{b} boards do not split into {groups} groups (or groups with the static workspace)")
 
     def dev32(key, required=True):
         if key not in state:
@@ -231,6 +239,12 @@ def run_forward_generic(
                                                layers, ck, cc, wptrs, bptrs, ptr(pw), ptr(pb),
                                                ptr(vw), ptr(vb), prec, ptr(logits), ptr(value),
                                                mask_mode, ptr(legal), fill, _lib.stream_ptr(dev))
+        elif groups > 1:
+            rc = lib.c6_forward_generic_grouped(x.data_ptr(), _lib.torch_dtype_code(x.dtype), groups,
+                                                b // groups, n, layers, ck, cc, wptrs, bptrs, ptr(pw),
+                                                ptr(pb), ptr(vw), ptr(vb), prec, workspace.data_ptr(),
+                                                workspace.numel(), ptr(logits), ptr(value), mask_mode,
+                                                ptr(legal), fill, _lib.stream_ptr(dev))
         else:
             rc = lib.c6_forward_generic(x.data_ptr(), _lib.torch_dtype_code(x.dtype), b, n, layers,
                                         ck, cc, wptrs, bptrs, ptr(pw), ptr(pb), ptr(vw), ptr(vb),
@@ -256,15 +270,16 @@ class PolicyValueNet(nn.Module):
     the boards whose decision is closer than that pass's rounding noise (the
     best free square leads the second best by less than ``cascade_threshold``
     standard deviations of the board's logits, default ``CASCADE_THRESHOLD``
-    = 0.02, or two others lie within twice that) once more with the corrected
-    arithmetic.  Over random networks it keeps the corrected mode's agreement
-    with the fp32 argmax to 0.01-0.02 % in the mean (99.2 %; a few such
-    networks fall just under 99 % in either mode) while about 6 % of their
-    boards are evaluated twice (a quarter, or all, when a network's logits
-    are nearly flat).  The modes it is made of have
-    to be asked for by name: ``"bf16"`` (every activation rounded to bf16
-    and nothing else, 98.8-98.9 % agreement) and ``"bf16f6"`` (bf16 MFMA plus
-    a correction pass on the activations' low-order part held in
+    = 0.02, or two others lie within twice that) once more with the low parts
+    of the activations and of the weights carried (``"bf16f6w"``: within 3e-4
+    of fp32).  Over random networks with the reference's initialisation its
+    argmax agrees with fp32's on 99.9 % of the boards (worst of 32 networks
+    99.7 %) while about 6 % of the boards are evaluated twice (a quarter, or
+    all, when a network's logits are nearly flat).  The modes it is made of
+    have to be asked for by name: ``"bf16"`` (every activation and weight
+    rounded to bf16 and nothing else, 98.8-98.9 % agreement), ``"bf16f6w"``
+    (on every board: twice the matrix work), and ``"bf16f6"`` (bf16 MFMA plus
+    a correction pass on the activations' low-order part alone, held in
     block-scaled fp6, on every board); also ``"fp32"`` and ``"fp16"``.
     """
 

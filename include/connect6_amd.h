@@ -38,8 +38,11 @@ extern "C" {
                             dropped, held as block-scaled fp6 (e2m3, one power-of-two scale per 32
                             channels), on the fp6 MFMA at four times the bf16 rate */
 #define C6_PREC_BF16C 4  /* cascade: every board in C6_PREC_BF16, then the boards whose decision
-                            is closer than the rounding noise again in C6_PREC_BF16F6; needs a
+                            is closer than the rounding noise again in C6_PREC_BF16F6W; needs a
                             workspace: c6_forward_cascade / c6_forward_boards_cascade */
+#define C6_PREC_BF16F6W 5 /* C6_PREC_BF16F6 plus, in the main pass, what the rounding of the
+                            weights to bf16 dropped (a second bf16 weight fragment per fragment,
+                            twice the bf16 matrix work): within 3e-4 relative L2 of fp32 */
 
 /* element types of caller tensors */
 #define C6_DT_F32 0
@@ -130,14 +133,14 @@ int c6_forward_boards(const int8_t *boards, const int8_t *player, const int8_t *
  * for that mode).  Replaces the same reference calls as they do (connect6/model.py:96-111,
  * connect6/history.py:276-303, connect6/train.py:730-748, :791-799).
  * First every board is evaluated with plain bf16 layer boundaries.  A board is evaluated again,
- * with the low-order correction of C6_PREC_BF16F6, when the rounding of the plain pass can change
+ * with the corrections of C6_PREC_BF16F6W, when the rounding of the plain pass can change
  * the move that an argmax picks (reference callers: connect6/benchmark.py:32,44,
  * connect6/evaluate.py:54, connect6/gui_cnn.py:43): when its largest logit among the free squares
  * (free as C6_MASK_LEGAL or the input planes say, whatever mask_mode writes) leads the second
  * largest by less than `threshold` standard deviations of the free squares' logits, or when two
  * other free squares lie within twice that of the largest.  Its logits, value and draw replace
  * the first ones.  threshold = 0 evaluates no board twice (results of C6_PREC_BF16), threshold < 0
- * every board (results of C6_PREC_BF16F6).  The plain pass's error on a difference of two logits
+ * every board (results of C6_PREC_BF16F6W).  The plain pass's error on a difference of two logits
  * is about 0.01 standard deviations of the logits; with threshold 0.02 random networks lose
  * 0.01-0.02 % of the corrected mode's agreement with fp32 in the mean while about 6 % of their
  * boards are evaluated twice.  A board's results do not depend on the other boards of the batch.
@@ -181,6 +184,25 @@ int c6_forward_generic(const void *x, int x_dtype, int64_t batch, int board, int
                        size_t workspace_bytes, float *logits, float *value, int mask_mode,
                        const uint8_t *legal, float fill, void *stream);
 
+/* c6_forward_generic for `groups` weight sets at once: one launch per layer for the whole
+ * ensemble.  Replaces: the non-default-architecture case of
+ * HistoricalPolicyEnsemble.forward_grouped (connect6/history.py:263-273: one grouped convolution
+ * per layer over the stacked parameters).
+ *   x        device [groups*boards_per_group,3,n,n]; board b uses weight set b / boards_per_group
+ *   conv_w[l] device fp32 [groups,Cout,Cin,k,k], conv_b[l] [groups,Cout] (the reference's stacked
+ *            layouts, connect6/history.py:224-240); pol_w [groups,C], pol_b [groups],
+ *            val_w [groups,C], val_b [groups]
+ *   workspace: c6_generic_workspace_bytes(groups*boards_per_group, ...) bytes
+ * Everything else as c6_forward_generic. */
+int c6_forward_generic_grouped(const void *x, int x_dtype, int64_t groups,
+                               int64_t boards_per_group, int board, int layers,
+                               const int *kernels, const int *channels,
+                               const float *const *conv_w, const float *const *conv_b,
+                               const float *pol_w, const float *pol_b, const float *val_w,
+                               const float *val_b, int prec, void *workspace,
+                               size_t workspace_bytes, float *logits, float *value, int mask_mode,
+                               const uint8_t *legal, float fill, void *stream);
+
 /* c6_forward_generic without a workspace argument, for callers that cannot allocate device
  * memory (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
  * It has no counterpart in the reference.  The layer-boundary activations go through a 16 MiB
@@ -188,7 +210,10 @@ int c6_forward_generic(const void *x, int x_dtype, int64_t batch, int board, int
  * ends); a batch whose c6_generic_workspace_bytes() exceeds that returns C6_EINVAL.  The call
  * allocates and frees nothing.  All calls on one GPU share that array: calls that overlap in
  * time on one GPU (different streams or threads) race; calls on one stream are safe back to
- * back.  Arguments and results as c6_forward_generic. */
+ * back.  The first call on a device looks the array's address up (hipGetSymbolAddress, which
+ * may load the code object and take the memory): a caller under graph capture makes one call
+ * per device outside the capture first; every later call only enqueues kernels.  Arguments and
+ * results as c6_forward_generic. */
 int c6_forward_generic_static(const void *x, int x_dtype, int64_t batch, int board, int layers,
                               const int *kernels, const int *channels,
                               const float *const *conv_w, const float *const *conv_b,

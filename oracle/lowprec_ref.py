@@ -1,6 +1,6 @@
 """fp32-PyTorch emulation of the arithmetic contracts of the 16-bit HIP modes that go beyond plain
-bf16 rounding: the bf16 + block-scaled-fp6 correction (``"bf16f6"``) and the decision rule of the
-cascade (``"bf16c"``).
+bf16 rounding: the bf16 + block-scaled-fp6 correction (``"bf16f6"``), the same with the weights'
+low part (``"bf16f6w"``), and the decision rule of the cascade (``"bf16c"``).
 
 TEST INFRASTRUCTURE ONLY -- the product (``connect6_amd``) never imports this.
 
@@ -24,7 +24,10 @@ function                   pinned by (tests/test_oracle.py)
 ``forward_bf16f6_emulated``  with ``lo_mask=0`` it equals ``torch_ref.forward_bf16_emulated``
                            bit for bit; with exact (unquantised) low-order parts and weights it
                            equals the forward with bf16 weights and unrounded activations to
-                           fp32 rounding; its distance to fp32 is below plain bf16's.
+                           fp32 rounding; its distance to fp32 is below plain bf16's;
+                           ``weights_lo`` with exact low-order parts equals the fp32 forward to
+                           2^-16 relative (the weights' second rounding), and with the e2m3
+                           roundings stays within 5e-4 of it.
 ``cascade_margin`` /       brute-force double-precision loop over the legal squares of small
 ``cascade_second_pass``    hand-made boards (ties, one or two legal squares, flat logits).
 =========================  ====================================================================
@@ -99,13 +102,16 @@ def lo_weight_copy(w: torch.Tensor) -> torch.Tensor:
 def forward_bf16f6_emulated(
     state: Mapping[str, torch.Tensor], x: torch.Tensor, lo_mask: int = 0xFE,
     act_scale: float = ACT_SCALE, exact_constant_plane: bool = True, exact_lo: bool = False,
+    weights_lo: bool = False,
 ) -> tuple[torch.Tensor, torch.Tensor]:
     """The ``"bf16f6"`` contract: as ``torch_ref.forward_bf16_emulated`` (bf16 weights and layer
     inputs, fp32 accumulation, fp32 bias + SiLU, last layer and heads in fp32), plus, for every
     3x3 layer l with bit l of ``lo_mask`` set, a second contraction of what the bf16 rounding of
     the layer's input dropped (``lo = a - bf16(a)``, block-scaled e2m3) with the e2m3 copy of
     the layer's weights.  ``exact_lo`` skips both e2m3 roundings (what the correction
-    approximates)."""
+    approximates).  ``weights_lo`` is the ``"bf16f6w"`` contract (the cascade's second pass): every
+    layer's bf16 input is also contracted with what the weights' rounding to bf16 dropped, itself
+    rounded to bf16 (``w = bf16(w) + bf16(w - bf16(w))`` to 16 mantissa bits)."""
     n = R._num_layers(state)
     c = float(act_scale)
     f = x
@@ -115,6 +121,8 @@ def forward_bf16f6_emulated(
         pad = w.shape[-1] // 2
         if i == 0:
             wq = R._bf16_round(w * c)
+            if weights_lo:
+                wq = wq + R._bf16_round(w * c - wq)
             xin = R._bf16_round(f)
             u = F.conv2d(xin, wq, b, padding=pad)
             if exact_constant_plane:
@@ -128,6 +136,8 @@ def forward_bf16f6_emulated(
             wq = R._bf16_round(w)
             hi = R._bf16_round(f)
             u = F.conv2d(hi, wq, b, padding=pad)
+            if weights_lo:
+                u = u + F.conv2d(hi, R._bf16_round(w - wq), None, padding=pad)
             if (lo_mask >> i) & 1:
                 lo = f - hi
                 if exact_lo:

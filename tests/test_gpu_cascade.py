@@ -1,5 +1,6 @@
 """The cascade mode ("bf16c") through the C ABI: every board in plain bf16, the boards whose
-decision is closer than the rounding noise again with the bf16 + fp6 correction.
+decision is closer than the rounding noise again with the low parts of activations and weights
+carried ("bf16f6w").
 
 What is checked: the two extremes of the threshold reproduce the two modes bit for bit; every
 output row is one of the two modes' rows and the choice follows the stated rule
@@ -45,7 +46,7 @@ def test_threshold_extremes_reproduce_the_two_modes(cuda):
     xd, ud = x.to(cuda), u.to(cuda)
     with torch.inference_mode():
         plain = make_model(cuda, st, "bf16")
-        fine = make_model(cuda, st, "bf16f6")
+        fine = make_model(cuda, st, "bf16f6w")
         for thr, other in ((0.0, plain), (-1.0, fine)):
             m = make_model(cuda, st, "bf16c", thr)
             for call in (lambda mm: mm(xd), lambda mm: mm.forward_masked(xd),
@@ -66,7 +67,7 @@ def test_rows_follow_the_rule_and_keep_the_gates_b4096(cuda, init):
     with torch.inference_mode():
         lo, vo = R.forward(st, x)
         lb, vb = make_model(cuda, st, "bf16")(xd)
-        lf, vf = make_model(cuda, st, "bf16f6")(xd)
+        lf, vf = make_model(cuda, st, "bf16f6w")(xd)
         m = make_model(cuda, st, "bf16c")              # default threshold
         lc, vc = m(xd)
     lb, lf, lc, vb, vf, vc = (t.cpu() for t in (lb, lf, lc, vb, vf, vc))
@@ -93,9 +94,11 @@ def test_rows_follow_the_rule_and_keep_the_gates_b4096(cuda, init):
     agree = argmax_agreement(masked(lc), masked(lo))
     agree_f6 = argmax_agreement(masked(lf), masked(lo))
     print(f"{init}: second pass {n2} of 4096 ({n2 / 4096:.3f}); argmax agreement cascade {agree:.4f}, "
-          f"bf16f6 {agree_f6:.4f}, bf16 {argmax_agreement(masked(lb), masked(lo)):.4f}")
+          f"second pass's arithmetic on every board {agree_f6:.4f}, bf16 {argmax_agreement(masked(lb), masked(lo)):.4f}")
     assert agree >= ARGMAX_MIN
-    assert agree >= agree_f6 - 0.002                   # what the threshold is allowed to cost
+    assert agree >= agree_f6 - 0.003                   # what the threshold is allowed to cost
+    if init == "reference":
+        assert agree >= 0.996                          # (measured 0.9988)
     if init == "reference":
         assert n2 <= 0.10 * 4096                       # the cascade pays: few boards go twice
 
@@ -190,7 +193,7 @@ def test_grouped_pack_equals_one_pack_per_model(cuda):
     first = _lib.packed_bytes(_lib.PREC_BF16)
     second_at = (first + 255) // 256 * 256
     for name, dtype in (("fp32", torch.float32), ("bf16", torch.bfloat16), ("fp16", torch.float16),
-                        ("bf16f6", torch.bfloat16), ("bf16c", torch.bfloat16)):
+                        ("bf16f6", torch.bfloat16), ("bf16f6w", torch.bfloat16), ("bf16c", torch.bfloat16)):
         ens = c6.HistoricalPolicyEnsemble(cps, cuda, dtype=dtype, precision=name)
         packed = ens._packed_weights()
         one = _lib.packed_bytes(ens._prec)
@@ -200,7 +203,7 @@ def test_grouped_pack_equals_one_pack_per_model(cuda):
         if name == "bf16c":
             spans = [(0, first - 32), (second_at, one)]
         else:
-            spans = [(0, one if name == "bf16f6" else one - 32)]
+            spans = [(0, one if name in ("bf16f6", "bf16f6w") else one - 32)]
         for m in range(5):
             alone = torch.empty(one, dtype=torch.uint8, device=cuda)
             pack_state(ens._model_state(m), ens._prec, alone)

@@ -43,6 +43,46 @@ def test_grouped_history_matches_individual_models_reference_test_shape(cuda):
             assert torch.all(value <= 1) and torch.all(value >= -1)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_grouped_generic_is_one_launch_per_layer_and_equals_model_by_model(cuda, dtype):
+    """An ensemble of a non-default architecture goes through c6_forward_generic_grouped (the
+    stacked parameters, every layer one launch for all models, as connect6/history.py:263-273) and
+    gives, bit for bit, what c6_forward_generic gives model by model."""
+    from connect6_amd.model import run_forward_generic
+
+    board, kernels, channels = 9, [5, 3, 1], [16, 24, 7]
+    cfg = {"architecture_version": 4, "kernels": kernels, "channels": channels}
+    cps = [c6.HistoricalCheckpoint(path=Path(f"m{i}.pt"), update=i + 1,
+                                   model_state=R.init_state(70 + i, "torch_default", kernels=kernels, channels=channels),
+                                   model_config=cfg, game_config={"board_size": board, "win_length": 6})
+           for i in range(5)]
+    ens = c6.HistoricalPolicyEnsemble(cps, cuda, dtype=dtype)
+    assert not ens.is_default_architecture
+    x = torch.randn(5, 7, 3, board, board, generator=torch.Generator().manual_seed(9))
+    x[:, :, :2] = (x[:, :, :2] > 0.8).float()
+    with torch.inference_mode():
+        grouped = ens.forward_grouped(x.to(cuda))
+        assert grouped.shape == (5, 7, board * board) and grouped.dtype == dtype
+        for i, cp in enumerate(cps):
+            single = run_forward_generic(x[i].to(cuda).to(dtype), ens._model_state(i), kernels, channels, ens._prec,
+                                         want_value=False)[0]
+            assert torch.equal(grouped[i], single.to(dtype)), i
+            want, _ = R.forward({k: v.to(dtype).float() for k, v in cp.model_state.items()}, x[i].to(dtype).float())
+            assert rel_l2(grouped[i].float().cpu(), want) <= (1e-5 if dtype == torch.float32 else 2e-2)
+    # argument checks of the grouped entry point
+    import ctypes
+
+    from connect6_amd import _lib
+    lib = c6.load()
+    ints = ctypes.c_int * 3
+    rc = lib.c6_forward_generic_grouped(None, 0, 0, 7, board, 3, ints(*kernels), ints(*channels), None, None, None,
+                                        None, None, None, 0, None, 0, None, None, 0, None, 0.0, None)
+    assert rc == -1 and b"groups" in lib.c6_last_error()
+    rc = lib.c6_forward_generic_grouped(None, 0, 5, 0, board, 3, ints(*kernels), ints(*channels), None, None, None,
+                                        None, None, None, 0, None, 0, None, None, 0, None, 0.0, None)
+    assert rc == 0                                          # no boards: nothing to do
+
+
 @pytest.mark.parametrize("board,kernels,channels", [(9, [5, 3, 1], [16, 24, 7]), (19, [7, 3], [5, 33])])
 def test_other_architectures_match_oracle_and_bruteforce(cuda, board, kernels, channels):
     st = R.init_state(11, "torch_default", kernels=kernels, channels=channels)

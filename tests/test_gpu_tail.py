@@ -122,11 +122,12 @@ def test_fused_selfplay_step_cfg4(cuda, prec):
     assert rel_l2(value[:1024], vo2) <= 2e-2
 
 
+@pytest.mark.parametrize("batch", [37, 44, 64])   # views not 16-byte aligned / whole groups of 32 planes + a partial one / whole groups
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_d4_expand_matches_oracle(cuda, dtype):
-    x = torch.randn(37, 3, 19, 19, generator=torch.Generator().manual_seed(2)).to(dtype)
+def test_d4_expand_matches_oracle(cuda, dtype, batch):
+    x = torch.randn(batch, 3, 19, 19, generator=torch.Generator().manual_seed(2)).to(dtype)
     views = c6.d4_expand(x.to(cuda)).cpu()
-    assert views.shape == (8, 37, 3, 19, 19)
+    assert views.shape == (8, batch, 3, 19, 19)
     assert torch.equal(views, R.d4_expand(x))
     for p in range(8):    # and the library routines the reference uses (train.py:222-230)
         k, flip = R.symmetry_for_phase(p)

@@ -30,10 +30,10 @@ def test_fused_kernels_stay_within_their_scratch_budget():
     arithmetic mode (headline and plain 16-bit modes tight, the others a ceiling)."""
     usage = _lib.resource_usage()
     fused = {name: u for name, u in usage.items() if "fused_forward_kernel" in name or "fused_pipe_kernel" in name}
-    assert len(fused) == 4
-    # bytes per lane; the pipelined kernels (bf16f6, bf16, fp16) keep two layers' accumulators live
-    # and still spill nothing: per-lane addresses are recomputed per board, not kept
-    limit = {"PrecBF16F6": 0, "PrecBF16E": 0, "PrecF16": 0, "PrecF32": 32}
+    assert len(fused) == 5
+    # bytes per lane; the pipelined kernels (bf16f6w, bf16f6, bf16, fp16) keep two layers'
+    # accumulators live and still spill nothing: per-lane addresses are recomputed per board, not kept
+    limit = {"PrecBF16F6W": 0, "PrecBF16F6E": 0, "PrecBF16E": 0, "PrecF16": 0, "PrecF32": 32}
     seen = set()
     for name, u in fused.items():
         for tag, cap in limit.items():
@@ -76,9 +76,14 @@ def test_packed_sizes_follow_the_layout():
     for cin, cout in zip((32, 32, 64, 64, 64, 96, 96), (32, 64, 64, 64, 96, 96, 96)):
         lo += ((9 * cin // 32 + 1) // 2) * (cout // 32) * 2
     assert _lib.packed_bytes(_lib.PREC_BF16F6) == (frags(8) + lo + 18 + fast1) * 1024 + tail
-    # cascade: the bf16 set, then (256-byte aligned) the bf16 + fp6 set
+    # ... and with the weights' low part: every fragment of the main pass twice (the first layer's
+    # two-plane copy too), the over-read padding and the rest as before
+    main = frags(8) - 24
+    fast1w = 2 * 23 * 3 + 8 + 4 * 3 * 4
+    assert _lib.packed_bytes(_lib.PREC_BF16F6W) == (2 * main + 24 + lo + 18 + fast1w) * 1024 + tail
+    # cascade: the bf16 set, then (256-byte aligned) the second pass's set
     first = (_lib.packed_bytes(_lib.PREC_BF16) + 255) // 256 * 256
-    assert _lib.packed_bytes(_lib.PREC_BF16C) == first + _lib.packed_bytes(_lib.PREC_BF16F6)
+    assert _lib.packed_bytes(_lib.PREC_BF16C) == first + _lib.packed_bytes(_lib.PREC_BF16F6W)
     assert _lib.cascade_workspace_bytes(0) == 16 and _lib.cascade_workspace_bytes(5) == 48
     with pytest.raises(ValueError):
         _lib.packed_bytes(9)
@@ -217,6 +222,8 @@ def test_precision_resolution_follows_torch_rules():
     assert model.resolve_precision() == _lib.PREC_F32
     model.precision = "bf16f6"
     assert model.resolve_precision() == _lib.PREC_BF16F6
+    model.precision = "bf16f6w"
+    assert model.resolve_precision() == _lib.PREC_BF16F6W
     model.precision = None
     # bf16 parameters (or bf16 autocast) select the cascade (plain bf16, corrected where the
     # decision is close); the two modes it is made of are by name only

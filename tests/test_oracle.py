@@ -365,6 +365,16 @@ def test_bf16f6_emulation_reduces_to_the_bf16_emulation_and_to_bf16_weights():
         e_plain = float((le - lw).norm() / lw.norm())
         e_f6 = float((l6 - lw).norm() / lw.norm())
         assert e_f6 < 0.25 * e_plain
+        # with the weights' low part as well ("bf16f6w"): exact low-order parts give the fp32
+        # forward up to the second rounding of the weights (2^-16 relative each), ...
+        # (input planes are bf16 operands of the first layer in every 16-bit mode: stones are exact)
+        lf, vf = R.forward(st, x.to(torch.bfloat16).float())
+        ly, vy = Q.forward_bf16f6_emulated(st, x, exact_lo=True, weights_lo=True, exact_constant_plane=False)
+        assert float((ly - lf).norm() / lf.norm()) < 3e-5 and float((vy - vf).norm() / vf.norm()) < 3e-5
+        # ... and the e2m3 roundings of the activations' low part leave a few 1e-4
+        lz, _ = Q.forward_bf16f6_emulated(st, x, weights_lo=True, exact_constant_plane=False)
+        e_w = float((lz - lf).norm() / lf.norm())
+        assert 2e-5 < e_w < 5e-4 and e_w < 0.1 * float((l6 - lf).norm() / lf.norm())
 
 
 def test_cascade_rule_against_a_plain_python_loop():
