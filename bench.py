@@ -28,7 +28,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per B=4096 launch of the fused kernel: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (one
 # run each), scaled by what the same counters read for a 256 MiB copy (x2.00 and x1.00); the
 # figures and commands are in profiles/fused_forward_<mode>_b4096.md.
-TRAFFIC_BYTES = {"bf16c": 42.7e6, "bf16f6": 33.7e6, "bf16": 31.2e6}
+TRAFFIC_BYTES = {"bf16c": 48.9e6, "bf16f6": 33.7e6, "bf16": 31.3e6}
 # The cascade: every board with plain bf16 layer boundaries, then the boards whose decision is
 # closer than the rounding noise again with the low parts of activations (fp6) and weights (bf16)
 # carried.  The fastest bf16-MFMA mode that meets the >= 99 % argmax gate, and it meets it with
