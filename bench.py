@@ -36,6 +36,11 @@ TRAFFIC_BYTES = {"bf16c": 48.9e6, "bf16f6": 33.7e6, "bf16": 31.3e6}
 HEADLINE = "bf16c"
 
 
+def _lib_names():
+    from connect6_amd import _lib
+    return _lib.PREC_BY_NAME
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -187,8 +192,10 @@ def main() -> int:
                 path=Path(f"model_update_{i + 1:08d}.pt"), update=i + 1,
                 model_state=c6.PolicyValueNet().state_dict(), model_config=cfg,
                 game_config={"board_size": 19, "win_length": 6}))
-        ens = c6.HistoricalPolicyEnsemble(cps, dev, dtype=torch.bfloat16,
-                                          precision=None if args.precision == "fp32" else args.precision)
+        # (a bf16 ensemble picks its own mode, as a caller's would: the cascade without a low part of
+        # the weights, which parameters held in bf16 do not have; any other mode is passed on)
+        ens_precision = None if args.precision in ("fp32", HEADLINE) else args.precision
+        ens = c6.HistoricalPolicyEnsemble(cps, dev, dtype=torch.bfloat16, precision=ens_precision)
         xg = x.view(8, B // 8, 3, 19, 19).to(torch.bfloat16)
 
         def timed(fn, steps=max(5, K // 2), warmup=3):
@@ -206,13 +213,13 @@ def main() -> int:
         out["grouped_g8"] = {
             "boards_per_s": B / tg, "ms": tg * 1e3, "ratio_to_single": (B / tg) / value,
             "workload": f"configs[2]: 8 weight sets x {B // 8} boards, one launch, bf16 in/out",
+            "precision_mode": {v: k for k, v in _lib_names().items()}[ens._prec],
         }
 
         # production shape of the history path (configs/train.yaml of the reference: up to 128
         # frozen models sharing 512 tables): weight traffic per board is 32x the G=8 case
         cps128 = [cps[i % 8] for i in range(128)]
-        ens128 = c6.HistoricalPolicyEnsemble(cps128, dev, dtype=torch.bfloat16,
-                                             precision=None if args.precision == "fp32" else args.precision)
+        ens128 = c6.HistoricalPolicyEnsemble(cps128, dev, dtype=torch.bfloat16, precision=ens_precision)
         xg128 = x[:512].view(128, 4, 3, 19, 19).to(torch.bfloat16)
         ens128.conv_weights, ens128.conv_biases, ens128.policy_weight, ens128.policy_bias   # (stack: host work + H2D)
         torch.cuda.synchronize()

@@ -20,9 +20,10 @@ _SOURCES = ("c6_forward.hip", "c6_tail.hip", "c6_generic.hip", "c6_env.hip", "c6
 _RESOURCES = _LIBDIR / "resource_usage.txt"   # registers, scratch and LDS of every kernel, written by build()
 
 # arithmetic modes (include/connect6_amd.h)
-PREC_F32, PREC_BF16, PREC_F16, PREC_BF16F6, PREC_BF16C, PREC_BF16F6W = 0, 1, 2, 3, 4, 5
+PREC_F32, PREC_BF16, PREC_F16, PREC_BF16F6, PREC_BF16C, PREC_BF16F6W, PREC_BF16C6 = 0, 1, 2, 3, 4, 5, 6
 PREC_BY_NAME = {"fp32": PREC_F32, "bf16": PREC_BF16, "fp16": PREC_F16, "bf16f6": PREC_BF16F6, "bf16c": PREC_BF16C,
-                "bf16f6w": PREC_BF16F6W}
+                "bf16f6w": PREC_BF16F6W, "bf16c6": PREC_BF16C6}
+CASCADES = (PREC_BF16C, PREC_BF16C6)   # the modes that go through the cascade entry points
 # cascade mode: a board is evaluated a second time (low parts of activations and weights carried) when its best free
 # square leads the second best by less than this many standard deviations of its logits, or two
 # other free squares lie within twice that.  The plain pass's error on a difference of two logits
@@ -184,10 +185,10 @@ def load() -> ctypes.CDLL:
     lib.c6_pack_weights_grouped.restype = i32
     lib.c6_pack_weights_grouped.argtypes = [ctypes.POINTER(vp), ctypes.POINTER(vp), vp, vp, vp, vp, i64, i32, vp,
                                             ctypes.c_size_t, vp]
-    lib.c6_forward_cascade.argtypes = [vp, i32, i64, i64, vp, ctypes.c_size_t, vp, i32, vp, i32, vp, f32,
+    lib.c6_forward_cascade.argtypes = [vp, i32, i64, i64, vp, ctypes.c_size_t, i32, vp, i32, vp, i32, vp, f32,
                                        vp, f32, vp, vp, f32, vp, ctypes.c_size_t, vp]
     lib.c6_forward_boards_cascade.restype = i32
-    lib.c6_forward_boards_cascade.argtypes = [vp, vp, vp, i64, vp, i32, i64, vp, vp, i32, vp, i32, f32, vp, f32,
+    lib.c6_forward_boards_cascade.argtypes = [vp, vp, vp, i64, vp, i32, i64, vp, i32, vp, i32, vp, i32, f32, vp, f32,
                                               vp, vp, f32, vp, ctypes.c_size_t, vp]
     ip = ctypes.POINTER(ctypes.c_int)
     lib.c6_generic_workspace_bytes.restype = i32

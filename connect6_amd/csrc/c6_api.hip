@@ -19,7 +19,7 @@ void set_error(const char *fmt, ...) {
 
 int dispatch_pack(int prec, const PackParams &pp, hipStream_t st);
 int dispatch_forward(int prec, const FwdParams &fp, hipStream_t st);
-int dispatch_cascade(const FwdParams &fp, float threshold, void *workspace, hipStream_t st);
+int dispatch_cascade(int prec, const FwdParams &fp, float threshold, void *workspace, hipStream_t st);
 size_t packed_bytes(int prec);
 int launch_mask(const void *, const uint8_t *, int, long long, uint32_t, void *, hipStream_t);
 int launch_sample(const float *, const uint8_t *, const float *, float, long long, long long *,
@@ -78,7 +78,7 @@ static int device_ok(const char *who) {
 
 static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 static int elem_bytes(int dt) { return dt == C6_DT_F32 ? 4 : ((dt == C6_DT_BF16 || dt == C6_DT_F16) ? 2 : 0); }
-static bool valid_prec(int p) { return p >= C6_PREC_F32 && p <= C6_PREC_BF16F6W; }
+static bool valid_prec(int p) { return p >= C6_PREC_F32 && p <= C6_PREC_BF16C6; }
 
 // the cascade's workspace argument, checked; `who` names the entry point in the message
 static int check_cascade_workspace(const char *who, long long boards, const void *workspace, size_t bytes) {
@@ -163,9 +163,9 @@ static int forward_planes(const char *who, const void *x, int x_dtype, int64_t g
                           const uint8_t *legal, float fill, const float *u, float temperature,
                           int64_t *actions, float *logprob, bool cascade, float threshold,
                           void *workspace, size_t workspace_bytes, void *stream) {
-  if (!valid_prec(prec) || (prec == C6_PREC_BF16C) != cascade) {
-    set_error("%s: precision mode %d is unknown or not served by this entry point (C6_PREC_BF16C "
-              "takes c6_forward_cascade, every other mode c6_forward)", who, prec);
+  if (!valid_prec(prec) || is_cascade(prec) != cascade) {
+    set_error("%s: precision mode %d is unknown or not served by this entry point (the cascade modes "
+              "take c6_forward_cascade, every other mode c6_forward)", who, prec);
     return C6_EINVAL;
   }
   if (elem_bytes(x_dtype) == 0 || elem_bytes(logits_dtype) == 0) {
@@ -228,7 +228,7 @@ static int forward_planes(const char *who, const void *x, int x_dtype, int64_t g
     if (rc != C6_OK) return rc;
   }
   C6_REQUIRE_DEVICE(who);
-  if (cascade) return dispatch_cascade(fp, threshold, workspace, static_cast<hipStream_t>(stream));
+  if (cascade) return dispatch_cascade(prec, fp, threshold, workspace, static_cast<hipStream_t>(stream));
   return dispatch_forward(prec, fp, static_cast<hipStream_t>(stream));
 }
 
@@ -251,12 +251,12 @@ int c6_cascade_workspace_bytes(int64_t boards, size_t *bytes) {
 }
 
 int c6_forward_cascade(const void *x, int x_dtype, int64_t groups, int64_t boards_per_group,
-                       const void *packed, size_t packed_stride, void *logits, int logits_dtype, float *value,
-                       int mask_mode, const uint8_t *legal, float fill, const float *u,
+                       const void *packed, size_t packed_stride, int prec, void *logits, int logits_dtype,
+                       float *value, int mask_mode, const uint8_t *legal, float fill, const float *u,
                        float temperature, int64_t *actions, float *logprob, float threshold,
                        void *workspace, size_t workspace_bytes, void *stream) {
   return forward_planes("c6_forward_cascade", x, x_dtype, groups, boards_per_group, packed, packed_stride,
-                        C6_PREC_BF16C, logits, logits_dtype, value, mask_mode, legal, fill, u, temperature,
+                        prec, logits, logits_dtype, value, mask_mode, legal, fill, u, temperature,
                         actions, logprob, true, threshold, workspace, workspace_bytes, stream);
 }
 
@@ -267,7 +267,7 @@ static int forward_states(const char *who, const int8_t *boards, const int8_t *p
                           int logits_dtype, float *value, int mask_mode, float fill, const float *u,
                           float temperature, int64_t *actions, float *logprob, bool cascade,
                           float threshold, void *workspace, size_t workspace_bytes, void *stream) {
-  if (!valid_prec(prec) || (prec == C6_PREC_BF16C) != cascade || elem_bytes(logits_dtype) == 0 || batch < 0 ||
+  if (!valid_prec(prec) || is_cascade(prec) != cascade || elem_bytes(logits_dtype) == 0 || batch < 0 ||
       batch > 0x7fffffffLL || view < 0 || view > 7 || num_states < 0) {
     set_error("%s: bad precision %d, batch %lld, states %lld or view %d", who, prec,
               (long long)batch, (long long)num_states, view);
@@ -322,7 +322,7 @@ static int forward_states(const char *who, const int8_t *boards, const int8_t *p
     if (rc != C6_OK) return rc;
   }
   C6_REQUIRE_DEVICE(who);
-  if (cascade) return dispatch_cascade(fp, threshold, workspace, static_cast<hipStream_t>(stream));
+  if (cascade) return dispatch_cascade(prec, fp, threshold, workspace, static_cast<hipStream_t>(stream));
   return dispatch_forward(prec, fp, static_cast<hipStream_t>(stream));
 }
 
@@ -339,12 +339,12 @@ int c6_forward_boards(const int8_t *boards, const int8_t *player, const int8_t *
 int c6_forward_boards_cascade(const int8_t *boards, const int8_t *player,
                               const int8_t *stones_left, int64_t num_states,
                               const int64_t *index, int view, int64_t batch, const void *packed,
-                              void *logits, int logits_dtype, float *value, int mask_mode, float fill,
+                              int prec, void *logits, int logits_dtype, float *value, int mask_mode, float fill,
                               const float *u, float temperature, int64_t *actions,
                               float *logprob, float threshold, void *workspace,
                               size_t workspace_bytes, void *stream) {
   return forward_states("c6_forward_boards_cascade", boards, player, stones_left, num_states, index, view,
-                        batch, packed, C6_PREC_BF16C, logits, logits_dtype, value, mask_mode, fill, u,
+                        batch, packed, prec, logits, logits_dtype, value, mask_mode, fill, u,
                         temperature, actions, logprob, true, threshold, workspace, workspace_bytes, stream);
 }
 

@@ -211,11 +211,15 @@ template <class P> struct Geo {
   static constexpr size_t PACKED_BYTES = TAIL_OFF + (size_t)TAIL_FLOATS * 4;
 };
 
-// Cascade mode (C6_PREC_BF16C): one packed set = the plain bf16 set, then (256-byte aligned)
-// the set of the same parameters for the second pass (bf16 + fp6 + the weights' low part).
-using PrecCascadeSecond = PrecBF16F6W;
+// Cascade modes: one packed set = the plain bf16 set, then (256-byte aligned) the set of the same
+// parameters for the second pass: bf16 + fp6 + the weights' low part (C6_PREC_BF16C), or, for
+// parameters that are exact in bf16 and have no low part, bf16 + fp6 (C6_PREC_BF16C6).
+constexpr bool is_cascade(int prec) { return prec == C6_PREC_BF16C || prec == C6_PREC_BF16C6; }
 constexpr size_t kCascadeSecondOffset = (Geo<PrecBF16>::PACKED_BYTES + 255) & ~(size_t)255;
-constexpr size_t kCascadePackedBytes = kCascadeSecondOffset + Geo<PrecCascadeSecond>::PACKED_BYTES;
+constexpr size_t cascade_packed_bytes(int prec) {
+  return kCascadeSecondOffset +
+         (prec == C6_PREC_BF16C ? Geo<PrecBF16F6W>::PACKED_BYTES : Geo<PrecBF16F6>::PACKED_BYTES);
+}
 // its workspace: int32 count (+ 3 words of padding), then one int32 per board
 constexpr size_t cascade_workspace_bytes(long long boards) { return (size_t)(16 + 4 * boards + 15) & ~(size_t)15; }
 

@@ -2152,12 +2152,12 @@ template <class P> static int launch_forward(const FwdParams &fp, hipStream_t st
 }
 
 int dispatch_pack(int prec, const PackParams &pp, hipStream_t st) {
-  if (prec == C6_PREC_BF16C) {  // both sets of the cascade
+  if (is_cascade(prec)) {  // both sets of the cascade
     const int rc = launch_pack<PrecBF16>(pp, st);
     if (rc != C6_OK) return rc;
     PackParams second = pp;
     second.packed = pp.packed + kCascadeSecondOffset;
-    return launch_pack<PrecCascadeSecond>(second, st);
+    return prec == C6_PREC_BF16C ? launch_pack<PrecBF16F6W>(second, st) : launch_pack<PrecBF16F6>(second, st);
   }
   switch (prec) {
     case C6_PREC_F32: return launch_pack<PrecF32>(pp, st);
@@ -2188,9 +2188,9 @@ __global__ void cascade_reset_kernel(int *count) {
 
 // Cascade: every board through the plain bf16 kernel, which lists the boards whose decision
 // margin is below `threshold`; then the listed boards through the kernel that also carries the
-// low parts of activations and weights, which overwrites their outputs.  Three launches on the caller's stream, no host synchronisation:
+// low parts of activations and (C6_PREC_BF16C) weights, which overwrites their outputs.  Three launches on the caller's stream, no host synchronisation:
 // the second kernel reads the length of the list from device memory.
-int dispatch_cascade(const FwdParams &fp, float threshold, void *workspace, hipStream_t st) {
+int dispatch_cascade(int prec, const FwdParams &fp, float threshold, void *workspace, hipStream_t st) {
   int *count = static_cast<int *>(workspace);
   hipLaunchKernelGGL(cascade_reset_kernel, dim3(1), dim3(64), 0, st, count);
   FwdParams first = fp;
@@ -2205,11 +2205,11 @@ int dispatch_cascade(const FwdParams &fp, float threshold, void *workspace, hipS
   second.redo_mode = kRedoConsume;
   second.redo_count = count;
   second.redo_list = count + 4;
-  return launch_forward<PrecCascadeSecond>(second, st);
+  return prec == C6_PREC_BF16C ? launch_forward<PrecBF16F6W>(second, st) : launch_forward<PrecBF16F6>(second, st);
 }
 
 size_t packed_bytes(int prec) {
-  if (prec == C6_PREC_BF16C) return kCascadePackedBytes;
+  if (is_cascade(prec)) return cascade_packed_bytes(prec);
   switch (prec) {
     case C6_PREC_F32: return Geo<PrecF32>::PACKED_BYTES;
     case C6_PREC_BF16: return Geo<PrecBF16>::PACKED_BYTES;

@@ -41,7 +41,7 @@ def _normalized_model_cfg(cfg: dict[str, Any]) -> dict[str, Any]:
 # precision="bf16", the corrections on every board as precision="bf16f6" / "bf16f6w".
 _PREC_OF_DTYPE = {
     torch.float32: _lib.PREC_F32,
-    torch.bfloat16: _lib.PREC_BF16C,
+    torch.bfloat16: _lib.PREC_BF16C6,   # (parameters held in bf16 have no low part: the second pass is bf16f6)
     torch.float16: _lib.PREC_F16,
 }
 
@@ -67,7 +67,7 @@ class HistoricalPolicyEnsemble:
     Input ``[MODELS, TABLES, 3, H, W]`` -> policy logits ``[MODELS, TABLES,
     H*W]`` in the ensemble dtype.  ``dtype`` selects the arithmetic as in the
     reference's ``_history_dtype`` (connect6/train.py:133-145): float32,
-    bfloat16 or float16.  bfloat16 runs the cascade (``"bf16c"``);
+    bfloat16 or float16.  bfloat16 runs the cascade (``"bf16c6"``);
     ``precision`` may name any other mode, e.g. ``"bf16"`` for the literal
     bf16 rounding of every activation.
 
@@ -210,7 +210,7 @@ class HistoricalPolicyEnsemble:
             return torch.empty((m, 0, self.action_size), dtype=self.dtype, device=self.device)
         if self.is_default_architecture:
             # (the cascade's entry point writes the logits in the ensemble's type itself)
-            direct = self._prec == _lib.PREC_BF16C and self.dtype != torch.float32
+            direct = self._prec in _lib.CASCADES and self.dtype != torch.float32
             logits, _, _, _ = run_forward(x.reshape(m * t, *expected_tail), self._packed_weights(),
                                           self._prec, m, t, want_value=False,
                                           logits_dtype=self.dtype if direct else torch.float32)

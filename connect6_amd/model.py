@@ -108,7 +108,7 @@ def run_forward(
     dev = x.device
     total = groups * boards_per_group
     x = x.contiguous()
-    if logits_dtype != torch.float32 and prec != _lib.PREC_BF16C:
+    if logits_dtype != torch.float32 and prec not in _lib.CASCADES:
         raise ValueError("only the cascade mode's entry point writes logits in another type than float32")
     logits = torch.empty((total, 361), dtype=logits_dtype, device=dev) if want_logits else None
     value = torch.empty((total,), dtype=torch.float32, device=dev) if want_value else None
@@ -134,11 +134,11 @@ def run_forward(
 
     stride = packed.numel() // groups if groups > 1 else packed.numel()
     with torch.cuda.device(dev):
-        if prec == _lib.PREC_BF16C:
+        if prec in _lib.CASCADES:
             ws = torch.empty(_lib.cascade_workspace_bytes(total) // 4, dtype=torch.int32, device=dev)
             rc = lib.c6_forward_cascade(
                 x.data_ptr(), _lib.torch_dtype_code(x.dtype), groups, boards_per_group, packed.data_ptr(),
-                stride, ptr(logits), _lib.torch_dtype_code(logits_dtype), ptr(value), mask_mode, ptr(legal), fill,
+                stride, prec, ptr(logits), _lib.torch_dtype_code(logits_dtype), ptr(value), mask_mode, ptr(legal), fill,
                 ptr(u), float(temperature), ptr(actions), ptr(logprob),
                 float(_lib.CASCADE_THRESHOLD if threshold is None else threshold),
                 ws.data_ptr(), ws.numel() * 4, _lib.stream_ptr(dev))
@@ -275,7 +275,9 @@ class PolicyValueNet(nn.Module):
     of fp32).  Over random networks with the reference's initialisation its
     argmax agrees with fp32's on 99.9 % of the boards (worst of 32 networks
     99.7 %) while about 6 % of the boards are evaluated twice (a quarter, or
-    all, when a network's logits are nearly flat).  The modes it is made of
+    all, when a network's logits are nearly flat; a module whose parameters
+    are held in bf16 runs ``"bf16c6"``, the same cascade without the weights'
+    low part, of which there is none).  The modes it is made of
     have to be asked for by name: ``"bf16"`` (every activation and weight
     rounded to bf16 and nothing else, 98.8-98.9 % agreement), ``"bf16f6w"``
     (on every board: twice the matrix work), and ``"bf16f6"`` (bf16 MFMA plus
@@ -363,12 +365,14 @@ class PolicyValueNet(nn.Module):
                 raise ValueError(
                     f"precision must be one of {sorted(_lib.PREC_BY_NAME)} or None, got {self.precision!r}"
                 ) from None
-        dtype = self.convs[0].weight.dtype
+        held = self.convs[0].weight.dtype
+        dtype = held
         if torch.is_autocast_enabled("cuda"):  # reference: train.py:126-130 wraps calls in autocast
             dtype = torch.get_autocast_dtype("cuda")
         if dtype == torch.bfloat16:
-            # the cascade: plain "bf16" alone misses the 99 % argmax agreement with fp32
-            return _lib.PREC_BF16C
+            # the cascade: plain "bf16" alone misses the 99 % argmax agreement with fp32.  Parameters
+            # that are held in bf16 have no low part for the second pass to carry.
+            return _lib.PREC_BF16C6 if held == torch.bfloat16 else _lib.PREC_BF16C
         if dtype == torch.float16:
             return _lib.PREC_F16
         return _lib.PREC_F32
@@ -599,12 +603,12 @@ def _forward_boards(
         return t.data_ptr() if t is not None else None
 
     with torch.cuda.device(dev):
-        if prec == _lib.PREC_BF16C:
+        if prec in _lib.CASCADES:
             ws = torch.empty(_lib.cascade_workspace_bytes(b) // 4, dtype=torch.int32, device=dev)
             thr = _lib.CASCADE_THRESHOLD if model.cascade_threshold is None else model.cascade_threshold
             rc = _lib.load().c6_forward_boards_cascade(
                 boards.data_ptr(), current_player.data_ptr(), stones_left.data_ptr(), n, ptr(index),
-                int(view), b, packed.data_ptr(), ptr(logits), _lib.DT_F32, value.data_ptr(),
+                int(view), b, packed.data_ptr(), prec, ptr(logits), _lib.DT_F32, value.data_ptr(),
                 _lib.MASK_INPUT if masked else _lib.MASK_NONE,
                 _FILL_LOWEST if fill is None else float(fill), ptr(u), float(temperature),
                 ptr(actions), ptr(logprob), float(thr), ws.data_ptr(), ws.numel() * 4, _lib.stream_ptr(dev))

@@ -40,6 +40,9 @@ extern "C" {
 #define C6_PREC_BF16C 4  /* cascade: every board in C6_PREC_BF16, then the boards whose decision
                             is closer than the rounding noise again in C6_PREC_BF16F6W; needs a
                             workspace: c6_forward_cascade / c6_forward_boards_cascade */
+#define C6_PREC_BF16C6 6  /* the cascade for parameters that are exact in bf16 (an ensemble or a
+                            module held in bf16): the weights have no low part, so the second
+                            pass is C6_PREC_BF16F6 */
 #define C6_PREC_BF16F6W 5 /* C6_PREC_BF16F6 plus, in the main pass, what the rounding of the
                             weights to bf16 dropped (a second bf16 weight fragment per fragment,
                             twice the bf16 matrix work): within 3e-4 relative L2 of fp32 */
@@ -129,8 +132,8 @@ int c6_forward_boards(const int8_t *boards, const int8_t *player, const int8_t *
                       const float *u, float temperature, int64_t *actions, float *logprob,
                       void *stream);
 
-/* c6_forward / c6_forward_boards in the cascade mode (C6_PREC_BF16C; `packed` holds sets packed
- * for that mode).  Replaces the same reference calls as they do (connect6/model.py:96-111,
+/* c6_forward / c6_forward_boards in a cascade mode (`prec` = C6_PREC_BF16C, or C6_PREC_BF16C6 for
+ * parameters that are exact in bf16; `packed` holds sets packed for that mode).  Replaces the same reference calls as they do (connect6/model.py:96-111,
  * connect6/history.py:276-303, connect6/train.py:730-748, :791-799).
  * First every board is evaluated with plain bf16 layer boundaries.  A board is evaluated again,
  * with the corrections of C6_PREC_BF16F6W, when the rounding of the plain pass can change
@@ -140,7 +143,8 @@ int c6_forward_boards(const int8_t *boards, const int8_t *player, const int8_t *
  * largest by less than `threshold` standard deviations of the free squares' logits, or when two
  * other free squares lie within twice that of the largest.  Its logits, value and draw replace
  * the first ones.  threshold = 0 evaluates no board twice (results of C6_PREC_BF16), threshold < 0
- * every board (results of C6_PREC_BF16F6W).  The plain pass's error on a difference of two logits
+ * every board (results of C6_PREC_BF16F6W; with C6_PREC_BF16C6, whose second pass leaves the
+ * weights' low part out because there is none, of C6_PREC_BF16F6).  The plain pass's error on a difference of two logits
  * is about 0.01 standard deviations of the logits; with threshold 0.02 random networks lose
  * 0.01-0.02 % of the corrected mode's agreement with fp32 in the mean while about 6 % of their
  * boards are evaluated twice.  A board's results do not depend on the other boards of the batch.
@@ -153,14 +157,14 @@ int c6_forward_boards(const int8_t *boards, const int8_t *player, const int8_t *
  * Three launches on `stream`, no synchronisation with the host. */
 int c6_cascade_workspace_bytes(int64_t boards, size_t *bytes);
 int c6_forward_cascade(const void *x, int x_dtype, int64_t groups, int64_t boards_per_group,
-                       const void *packed, size_t packed_stride, void *logits, int logits_dtype,
+                       const void *packed, size_t packed_stride, int prec, void *logits, int logits_dtype,
                        float *value, int mask_mode, const uint8_t *legal, float fill, const float *u,
                        float temperature, int64_t *actions, float *logprob, float threshold,
                        void *workspace, size_t workspace_bytes, void *stream);
 int c6_forward_boards_cascade(const int8_t *boards, const int8_t *player,
                               const int8_t *stones_left, int64_t num_states,
                               const int64_t *index, int view, int64_t batch, const void *packed,
-                              void *logits, int logits_dtype, float *value, int mask_mode, float fill,
+                              int prec, void *logits, int logits_dtype, float *value, int mask_mode, float fill,
                               const float *u, float temperature, int64_t *actions,
                               float *logprob, float threshold, void *workspace,
                               size_t workspace_bytes, void *stream);

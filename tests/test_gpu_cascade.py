@@ -103,6 +103,38 @@ def test_rows_follow_the_rule_and_keep_the_gates_b4096(cuda, init):
         assert n2 <= 0.10 * 4096                       # the cascade pays: few boards go twice
 
 
+def test_cascade_for_parameters_held_in_bf16(cuda):
+    """"bf16c6": the cascade whose second pass leaves the weights' low part out, for parameters that
+    are exact in bf16 (what a bf16 module or ensemble holds).  Its extremes are bf16 and bf16f6;
+    on such parameters "bf16c" lists the same boards and its second pass multiplies the
+    activations with low parts that are all zero -- except in the first layer, whose weights are
+    rounded after the activation scale is folded in: that is all that separates the two."""
+    st = {k: v.to(torch.bfloat16).float() for k, v in R.init_state(1234, "reference").items()}
+    x, legal = gen_boards(1500, 200, 2025)
+    xd = x.to(cuda)
+    with torch.inference_mode():
+        plain, fine = make_model(cuda, st, "bf16"), make_model(cuda, st, "bf16f6")
+        for thr, other in ((0.0, plain), (-1.0, fine)):
+            m = make_model(cuda, st, "bf16c6", thr)
+            got, want = m.forward_masked(xd), other.forward_masked(xd)
+            assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+        a, b = make_model(cuda, st, "bf16c6"), make_model(cuda, st, "bf16c")
+        la, va = a.forward_masked(xd)
+        lb, vb = b.forward_masked(xd)
+        assert 0 < second_pass(a) == second_pass(b) < 150
+        once = (la == make_model(cuda, st, "bf16").forward_masked(xd)[0]).all(1)
+        assert torch.equal(la[once], lb[once]) and int((~once).sum()) <= second_pass(a)
+        assert rel_l2(la[~once].cpu().masked_fill(~legal[~once.cpu()], 0), lb[~once].cpu().masked_fill(~legal[~once.cpu()], 0)) <= 3e-3
+        assert rel_l2(va, vb) <= 3e-3
+        # a module that holds its parameters in bf16 picks it by itself
+        held = c6.PolicyValueNet().to(cuda).eval()
+        held.load_state_dict(st)
+        held = held.to(torch.bfloat16)
+        assert held.resolve_precision() == _lib.PREC_BF16C6
+        lh, vh = held.forward_masked(xd.to(torch.bfloat16))
+        assert torch.equal(lh, la) and torch.equal(vh, va)
+
+
 def test_a_boards_result_does_not_depend_on_the_batch(cuda):
     st = R.init_state(11, "reference")
     x, legal = gen_boards(1000, 200, 77)
@@ -168,8 +200,8 @@ def test_cascade_entry_points_check_their_workspace(cuda):
     x = gen_boards(100, 200, 1)[0].to(cuda)
     out = torch.empty(100, 361, device=cuda)
     small = torch.empty(16, dtype=torch.int32, device=cuda)
-    args = (x.data_ptr(), _lib.DT_F32, 1, 100, packed.data_ptr(), packed.numel(), out.data_ptr(), _lib.DT_F32, None,
-            _lib.MASK_NONE, None, 0.0, None, 1.0, None, None, 0.03)
+    args = (x.data_ptr(), _lib.DT_F32, 1, 100, packed.data_ptr(), packed.numel(), _lib.PREC_BF16C, out.data_ptr(),
+            _lib.DT_F32, None, _lib.MASK_NONE, None, 0.0, None, 1.0, None, None, 0.03)
     rc = lib.c6_forward_cascade(*args, small.data_ptr(), small.numel() * 4, _lib.stream_ptr(cuda))
     assert rc == -1 and b"workspace" in lib.c6_last_error()
     rc = lib.c6_forward_cascade(*args, None, 1 << 20, _lib.stream_ptr(cuda))
@@ -193,14 +225,15 @@ def test_grouped_pack_equals_one_pack_per_model(cuda):
     first = _lib.packed_bytes(_lib.PREC_BF16)
     second_at = (first + 255) // 256 * 256
     for name, dtype in (("fp32", torch.float32), ("bf16", torch.bfloat16), ("fp16", torch.float16),
-                        ("bf16f6", torch.bfloat16), ("bf16f6w", torch.bfloat16), ("bf16c", torch.bfloat16)):
+                        ("bf16f6", torch.bfloat16), ("bf16f6w", torch.bfloat16), ("bf16c", torch.bfloat16),
+                        ("bf16c6", torch.bfloat16)):
         ens = c6.HistoricalPolicyEnsemble(cps, cuda, dtype=dtype, precision=name)
         packed = ens._packed_weights()
         one = _lib.packed_bytes(ens._prec)
         assert packed.shape == (5, one)
         # bytes every mode defines: all fragments and the fp32 tail; the eight scale words behind
         # it only where a low-order copy exists; the cascade's alignment gap not at all
-        if name == "bf16c":
+        if name in ("bf16c", "bf16c6"):
             spans = [(0, first - 32), (second_at, one)]
         else:
             spans = [(0, one if name in ("bf16f6", "bf16f6w") else one - 32)]

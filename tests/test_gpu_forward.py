@@ -294,7 +294,7 @@ def test_grouped_g8_bf16_cfg3(cuda, precision):
     torch.set_num_threads(16)
     cps = _checkpoints(8)
     ens = c6.HistoricalPolicyEnsemble(cps, cuda, dtype=torch.bfloat16, precision=precision)
-    assert ens._prec == _lib.PREC_BY_NAME[precision or "bf16c"]
+    assert ens._prec == _lib.PREC_BY_NAME[precision or "bf16c6"]   # (held in bf16: no low part of the weights)
     x, legal = gen_boards(4096, 200, 2025)
     xg, lg = x.view(8, 512, 3, 19, 19), legal.view(8, 512, 361)
     with torch.inference_mode():

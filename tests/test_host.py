@@ -84,6 +84,8 @@ def test_packed_sizes_follow_the_layout():
     # cascade: the bf16 set, then (256-byte aligned) the second pass's set
     first = (_lib.packed_bytes(_lib.PREC_BF16) + 255) // 256 * 256
     assert _lib.packed_bytes(_lib.PREC_BF16C) == first + _lib.packed_bytes(_lib.PREC_BF16F6W)
+    # ... or, for parameters that are exact in bf16, the bf16 + fp6 set
+    assert _lib.packed_bytes(_lib.PREC_BF16C6) == first + _lib.packed_bytes(_lib.PREC_BF16F6)
     assert _lib.cascade_workspace_bytes(0) == 16 and _lib.cascade_workspace_bytes(5) == 48
     with pytest.raises(ValueError):
         _lib.packed_bytes(9)
@@ -102,13 +104,17 @@ def test_entry_points_reject_bad_arguments_before_touching_the_device():
     assert lib.c6_forward(None, 0, 1, 4, None, 0, _lib.PREC_BF16C, None, None, 0, None, 0.0, None, 1.0, None, None,
                           None) == -1
     assert b"c6_forward_cascade" in lib.c6_last_error()
-    assert lib.c6_forward_cascade(None, 0, 1, 4, None, 0, None, 0, None, 0, None, 0.0, None, 1.0, None, None, 0.03,
+    C, C6 = _lib.PREC_BF16C, _lib.PREC_BF16C6
+    assert lib.c6_forward_cascade(None, 0, 1, 4, None, 0, C, None, 0, None, 0, None, 0.0, None, 1.0, None, None, 0.03,
                                   None, 0, None) == -1
-    assert lib.c6_forward_cascade(None, 0, 1, 0, None, 0, None, 0, None, 0, None, 0.0, None, 1.0, None, None, 0.03,
+    assert lib.c6_forward_cascade(None, 0, 1, 0, None, 0, C6, None, 0, None, 0, None, 0.0, None, 1.0, None, None, 0.03,
                                   None, 0, None) == 0
-    assert lib.c6_forward_cascade(None, 0, 1, 4, None, 0, None, 9, None, 0, None, 0.0, None, 1.0, None, None, 0.03,
+    assert lib.c6_forward_cascade(None, 0, 1, 4, None, 0, C, None, 9, None, 0, None, 0.0, None, 1.0, None, None, 0.03,
                                   None, 0, None) == -1                  # unknown element type of the logits
-    assert lib.c6_forward_boards_cascade(None, None, None, 4, None, 0, 4, None, None, 0, None, 1, 0.0, None, 1.0,
+    assert lib.c6_forward_cascade(None, 0, 1, 4, None, 0, _lib.PREC_BF16, None, 0, None, 0, None, 0.0, None, 1.0, None,
+                                  None, 0.03, None, 0, None) == -1      # not a cascade mode
+    assert b"c6_forward" in lib.c6_last_error()
+    assert lib.c6_forward_boards_cascade(None, None, None, 4, None, 0, 4, None, C, None, 0, None, 1, 0.0, None, 1.0,
                                          None, None, 0.03, None, 0, None) == -1
     assert lib.c6_pack_weights_grouped(None, None, None, None, None, None, 0, 1, None, 0, None) == -1
     size = ctypes.c_size_t(0)
@@ -227,7 +233,9 @@ def test_precision_resolution_follows_torch_rules():
     model.precision = None
     # bf16 parameters (or bf16 autocast) select the cascade (plain bf16, corrected where the
     # decision is close); the two modes it is made of are by name only
-    assert model.to(torch.bfloat16).resolve_precision() == _lib.PREC_BF16C
+    # (under bf16 autocast, which needs the GPU, fp32 parameters select "bf16c": the GPU tests hold
+    # that; parameters held in bf16 have no low part for the second pass to carry)
+    assert model.to(torch.bfloat16).resolve_precision() == _lib.PREC_BF16C6
     assert model.to(torch.float16).resolve_precision() == _lib.PREC_F16
     model.precision = "bf16"
     assert model.resolve_precision() == _lib.PREC_BF16
@@ -262,7 +270,7 @@ def test_history_ensemble_construction_and_validation():
     assert ens.policy_weight.shape == (2, 1, 96, 1, 1) and ens.policy_bias.shape == (2, 1)
     assert ens._prec == _lib.PREC_F32
     ens16 = c6.HistoricalPolicyEnsemble(cps, torch.device("cpu"), dtype=torch.bfloat16)
-    assert ens16._prec == _lib.PREC_BF16C and ens16.conv_weights[3].dtype == torch.bfloat16
+    assert ens16._prec == _lib.PREC_BF16C6 and ens16.conv_weights[3].dtype == torch.bfloat16
     assert c6.HistoricalPolicyEnsemble(cps, torch.device("cpu"), dtype=torch.bfloat16, precision="bf16")._prec == _lib.PREC_BF16
     # compile keys are ignored when comparing architectures (history.py:69-73)
     cps[1].model_config["compile"] = True
