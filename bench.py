@@ -103,8 +103,8 @@ def main() -> int:
     kernel_name = {"fp32": "fused_forward_kernel<fp32>"}.get(args.precision, f"fused_pipe_kernel<{args.precision}>")
     cascade = None
     if args.precision == "bf16c":
-        # HIP events bracket the whole step: the reset of the list, the bf16 kernel over all
-        # boards, the bf16 + fp6 kernel over the listed ones.  The first pass alone is timed with
+        # HIP events bracket the whole step: the bf16 kernel over all boards, then the kernel
+        # that carries the low parts over the listed ones.  The first pass alone is timed with
         # threshold 0 (no board listed; the second kernel still starts and finds nothing).
         kernel_name = "fused_pipe_kernel<bf16> over all boards + fused_pipe_kernel<bf16f6w> over the listed boards"
         twice = int(model.cascade_stats["second_pass"].item())

@@ -165,7 +165,10 @@ template <class P> struct Geo {
   // directly, so the input never sits in registers (or, under register pressure, in scratch).
   static constexpr int NEXT_IN_OFF = TAIL_LDS_OFF + (kBiasTotal + 2 * kHeadC + 4) * 4;
   static constexpr int NEXT_IN_AUX = 1084, NEXT_IN_BYTES_AT = 1088;
-  static constexpr int LDS_BYTES = P::PIPE ? NEXT_IN_OFF + (NEXT_IN_BYTES_AT + 384) * 4 : TAIL_LDS_OFF;
+  // ... and, for the cascade's second pass, the running sums of the first pass's per-workgroup
+  // counts of listed boards (kCascadeMaxRuns + 1 ints)
+  static constexpr int RUNS_OFF = NEXT_IN_OFF + (NEXT_IN_BYTES_AT + 384) * 4;
+  static constexpr int LDS_BYTES = P::PIPE ? RUNS_OFF + (1024 + 1 + 3) * 4 : TAIL_LDS_OFF;
 
   static constexpr int layer_steps(int l) { return l == 0 ? STEPS1 : 9 * kCinArr[l] / KSTEP; }
   static constexpr int layer_frags(int l) { return layer_steps(l) * (kCoutArr[l] / 32) * W; }
@@ -220,8 +223,17 @@ constexpr size_t cascade_packed_bytes(int prec) {
   return kCascadeSecondOffset +
          (prec == C6_PREC_BF16C ? Geo<PrecBF16F6W>::PACKED_BYTES : Geo<PrecBF16F6>::PACKED_BYTES);
 }
-// its workspace: int32 count (+ 3 words of padding), then one int32 per board
-constexpr size_t cascade_workspace_bytes(long long boards) { return (size_t)(16 + 4 * boards + 15) & ~(size_t)15; }
+// Its workspace.  Every workgroup of the first pass keeps the list of its own boards that need the
+// second pass (it evaluates one contiguous run of boards; its list has room for all of them) and
+// writes their number when its run is done: no atomic operation, and nothing to clear before a
+// call.  The second pass sums the counts up (every workgroup for itself) and deals the listed boards
+// out evenly.  Layout, in int32: [0] boards listed in all (written by the second pass, for the
+// caller), [4, 4 + kCascadeMaxRuns) the counts per run, then the lists, `per` entries per run
+// (runs x per <= boards + runs).
+constexpr int kCascadeMaxRuns = 1024;   // workgroups of the first pass = compute units, at most
+constexpr size_t cascade_workspace_bytes(long long boards) {
+  return (size_t)(16 + 4 * (long long)kCascadeMaxRuns + 4 * (boards + kCascadeMaxRuns) + 15) & ~(size_t)15;
+}
 
 constexpr int bias_offset(int l) {
   int s = 0;
@@ -257,8 +269,11 @@ struct FwdParams {
   // cascade (C6_PREC_BF16C; pipelined kernel only)
   int redo_mode = kRedoNone;      // kRedoDetect: first pass, kRedoConsume: second pass
   float redo_threshold = 0.0f;    // first pass: < 0 = every board goes on the list
-  int *redo_count = nullptr;      // number of list entries (device memory)
-  int *redo_list = nullptr;       // boards for the second pass (device memory, one int per board)
+  int *redo_count = nullptr;      // boards listed in all (device memory; the second pass writes it)
+  int *redo_counts = nullptr;     // boards listed by run r of the first pass
+  int *redo_list = nullptr;       // run r's list starts at entry r * redo_per
+  int redo_runs = 0;              // workgroups (runs of boards) of the first pass
+  int redo_per = 0;               // boards per run of the first pass
 };
 
 struct PackParams {

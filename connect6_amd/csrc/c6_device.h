@@ -67,6 +67,21 @@ __device__ __forceinline__ float wave_inclusive_sum(float v) {
   return v;
 }
 
+// the same for integers
+__device__ __forceinline__ int wave_inclusive_sum_i(int v) {
+  auto shifted = [](int x, auto ctrl, auto rows) {
+    return __builtin_amdgcn_update_dpp(0, x, decltype(ctrl)::value, decltype(rows)::value, 0xF, false);
+  };
+  using std::integral_constant;
+  v += shifted(v, integral_constant<int, 0x111>{}, integral_constant<int, 0xF>{});  // row_shr:1
+  v += shifted(v, integral_constant<int, 0x112>{}, integral_constant<int, 0xF>{});  // row_shr:2
+  v += shifted(v, integral_constant<int, 0x114>{}, integral_constant<int, 0xF>{});  // row_shr:4
+  v += shifted(v, integral_constant<int, 0x118>{}, integral_constant<int, 0xF>{});  // row_shr:8
+  v += shifted(v, integral_constant<int, 0x142>{}, integral_constant<int, 0xA>{});  // row_bcast:15 -> rows 1, 3
+  v += shifted(v, integral_constant<int, 0x143>{}, integral_constant<int, 0xC>{});  // row_bcast:31 -> rows 2, 3
+  return v;
+}
+
 __device__ __forceinline__ float wave_min(float v) {
   return __builtin_bit_cast(float, wave_allreduce_bits(__builtin_bit_cast(int, v), [](int a, int b) {
     return __builtin_bit_cast(int, fminf(__builtin_bit_cast(float, a), __builtin_bit_cast(float, b)));

@@ -1252,19 +1252,65 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
   // workgroups of one XCD (workgroup i runs on XCD i % 8) cover one contiguous eighth of the
   // batch: with several weight sets an XCD's L2 then holds only the sets of its own boards, and
   // consecutive boards of a workgroup mostly reuse the set it has just streamed.
-  // Cascade, second pass (prm.redo_mode == kRedoConsume): the boards to evaluate are the entries
-  // of the list the first pass wrote, their number sits in device memory.
-  const bool from_list = prm.redo_mode == kRedoConsume;
-  const unsigned n_items = from_list ? (unsigned)*prm.redo_count : (unsigned)prm.total_boards;
-  auto board_of = [&](unsigned i) { return from_list ? (unsigned)prm.redo_list[i] : i; };
+  // Cascade, second pass (prm.redo_mode == kRedoConsume): the boards to evaluate are the ones the
+  // first pass listed, run by run (run r: redo_counts[r] boards at redo_list[r * redo_per ...]).
+  // Every workgroup sums the counts up for itself -- `runs[r]` = boards listed by the runs before
+  // r, `runs[redo_runs]` = all of them -- and the listed boards, numbered in that order, are dealt
+  // out like the boards of any batch.
+  // (compiled into the kernels that can be a cascade's passes only: the first pass is plain bf16,
+  // the second one of the modes that carry low parts)
+  constexpr bool kCanDetect = P::ID == C6_PREC_BF16, kCanConsume = P::LO6 != 0;
+  const bool from_list = kCanConsume && prm.redo_mode == kRedoConsume;
+  const bool detect = kCanDetect && prm.redo_mode == kRedoDetect;
+  int *runs = reinterpret_cast<int *>(smem + G::RUNS_OFF);
+  unsigned n_items = (unsigned)prm.total_boards;
+  if (from_list) {
+    int *part = reinterpret_cast<int *>(red);   // the four waves' sums
+    int before = 0;
+    for (int r0 = 0; r0 < prm.redo_runs; r0 += THREADS) {
+      const int r = r0 + tid;
+      const int c = r < prm.redo_runs ? prm.redo_counts[r] : 0;
+      const int incl = wave_inclusive_sum_i(c);
+      if (lane == 63) part[wave] = incl;
+      __syncthreads();
+      int lower = before;
+#pragma unroll
+      for (int w = 0; w < NWAVES; ++w) {
+        lower += w < wave ? part[w] : 0;
+        before += part[w];
+      }
+      if (r < prm.redo_runs) runs[r] = lower + incl - c;
+      __syncthreads();
+    }
+    if (tid == 0) {
+      runs[prm.redo_runs] = before;
+      if (blockIdx.x == 0) *prm.redo_count = before;   // for the caller: boards evaluated twice
+    }
+    __syncthreads();
+    n_items = (unsigned)before;
+  }
+  // listed board i: the run r with runs[r] <= i < runs[r + 1] (a bisection; the same in every thread)
+  auto board_of = [&](unsigned i) {
+    if (!from_list) return i;
+    int lo = 0, hi = prm.redo_runs;
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if ((unsigned)runs[mid] <= i) lo = mid; else hi = mid;
+    }
+    return (unsigned)prm.redo_list[(size_t)lo * prm.redo_per + (i - (unsigned)runs[lo])];
+  };
   const unsigned per = (n_items + gridDim.x - 1) / gridDim.x;
   const unsigned xcds = (gridDim.x % 8 == 0) ? 8 : 1;
   const unsigned run = (blockIdx.x % xcds) * (gridDim.x / xcds) + blockIdx.x / xcds;
   // (board counts fit 31 bits, host-checked; a run beyond the last board starts past n_items)
   const unsigned long long first_item = (unsigned long long)run * per;
-  if (first_item >= n_items) return;
+  if (first_item >= n_items) {
+    if (detect && tid == 0) prm.redo_counts[run] = 0;   // (a run without boards lists none)
+    return;
+  }
   unsigned it = (unsigned)first_item;  // position in the run of boards; `b` below is the board itself
   const unsigned it_end = n_items - it > per ? it + per : n_items;
+  int listed = 0;                      // cascade, first pass: boards of this run listed so far (wave 1 counts)
   [[maybe_unused]] const unsigned it_first = it;
   v4i r1[L1Pipe<P>::D][1];
   // (the first layer's weight ring is filled, a board ahead, with the stream for a constant
@@ -1586,7 +1632,7 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
         if (prm.logprob != nullptr) prm.logprob[b] = lp;
       }
     }
-    if (prm.redo_mode == kRedoDetect && wave == 1) {
+    if (detect && wave == 1) {
       // Cascade, first pass: a board whose best free square leads the second best by less than
       // the threshold (in standard deviations of its free squares' logits) is put on the list
       // of boards that the second pass evaluates again with the corrected arithmetic.
@@ -1596,11 +1642,15 @@ __global__ __launch_bounds__(256) void fused_pipe_kernel(const FwdParams prm) {
       asm volatile("" : "+v"(lane_here));
       const bool again = wave_margin_below(
           lane_here, tau, [&](int i) { return lgt[i]; }, [&](int i) { return (occ[i] & 2) == 0; });
-      if (lane == 0 && again) prm.redo_list[atomicAdd(prm.redo_count, 1)] = (int)b;
+      if (again) {   // (wave-uniform)
+        if (lane == 0) prm.redo_list[(size_t)run * prm.redo_per + listed] = (int)b;
+        ++listed;
+      }
     }
     C6_MARK(20);
     b = bn;
   }
+  if (detect && wave == 1 && lane == 0) prm.redo_counts[run] = listed;
 }
 
 // ------------------------------------------------------------------------
@@ -2182,29 +2232,55 @@ int dispatch_forward(int prec, const FwdParams &fp, hipStream_t st) {
   return C6_EINVAL;
 }
 
-__global__ void cascade_reset_kernel(int *count) {
-  if (threadIdx.x == 0) *count = 0;
+// compute units of the current device (the grid of the persistent kernels)
+static int device_cus(int &cus) {
+  static thread_local int known_dev = -1, known_cus = 0;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e == hipSuccess && dev != known_dev) {
+    int n = 0;
+    e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e == hipSuccess) {
+      known_dev = dev;
+      known_cus = n;
+    }
+  }
+  if (e != hipSuccess) {
+    set_error("device query failed: %s", hipGetErrorString(e));
+    return C6_ELAUNCH;
+  }
+  cus = known_cus > 0 ? known_cus : 256;
+  return C6_OK;
 }
 
-// Cascade: every board through the plain bf16 kernel, which lists the boards whose decision
-// margin is below `threshold`; then the listed boards through the kernel that also carries the
-// low parts of activations and (C6_PREC_BF16C) weights, which overwrites their outputs.  Three launches on the caller's stream, no host synchronisation:
-// the second kernel reads the length of the list from device memory.
+// Cascade: every board through the plain bf16 kernel, whose workgroups list those of their boards
+// whose decision margin is below `threshold`; then the listed boards through the kernel that also
+// carries the low parts of activations and (C6_PREC_BF16C) weights, which overwrites their
+// outputs.  Two launches on the caller's stream, no host synchronisation, no atomic operation and
+// nothing to clear: the second kernel reads how many boards each workgroup of the first listed.
 int dispatch_cascade(int prec, const FwdParams &fp, float threshold, void *workspace, hipStream_t st) {
-  int *count = static_cast<int *>(workspace);
-  hipLaunchKernelGGL(cascade_reset_kernel, dim3(1), dim3(64), 0, st, count);
+  int cus = 0;
+  int rc = device_cus(cus);
+  if (rc != C6_OK) return rc;
+  const long long runs = cus < fp.total_boards ? cus : fp.total_boards;   // = the first kernel's grid
+  if (runs > kCascadeMaxRuns) {
+    set_error("cascade: %lld workgroups exceed the %d the workspace layout provides for", runs, kCascadeMaxRuns);
+    return C6_EINVAL;
+  }
+  int *ws = static_cast<int *>(workspace);
   FwdParams first = fp;
   first.redo_mode = kRedoDetect;
   first.redo_threshold = threshold;
-  first.redo_count = count;
-  first.redo_list = count + 4;
-  int rc = launch_forward<PrecBF16>(first, st);
+  first.redo_count = ws;
+  first.redo_counts = ws + 4;
+  first.redo_list = ws + 4 + kCascadeMaxRuns;
+  first.redo_runs = (int)runs;
+  first.redo_per = (int)((fp.total_boards + runs - 1) / runs);
+  rc = launch_forward<PrecBF16>(first, st);
   if (rc != C6_OK) return rc;
-  FwdParams second = fp;
+  FwdParams second = first;
   second.packed = fp.packed + kCascadeSecondOffset;
   second.redo_mode = kRedoConsume;
-  second.redo_count = count;
-  second.redo_list = count + 4;
   return prec == C6_PREC_BF16C ? launch_forward<PrecBF16F6W>(second, st) : launch_forward<PrecBF16F6>(second, st);
 }
 

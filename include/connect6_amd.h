@@ -152,9 +152,11 @@ int c6_forward_boards(const int8_t *boards, const int8_t *player, const int8_t *
  *              C6_DT_F16; may be NULL): a bf16 / fp16 ensemble gets its logits rounded once (to
  *              nearest even, as Tensor.to does) by the kernel instead of by a cast behind it;
  *              `fill` is converted the same way
- *   workspace  device, c6_cascade_workspace_bytes(boards) bytes, 16-byte aligned; after the
+ *   workspace  device, c6_cascade_workspace_bytes(boards) bytes, 16-byte aligned, contents
+ *              arbitrary (nothing has to be cleared: every workgroup of the first pass lists its
+ *              own boards and writes how many, the second pass adds the counts up); after the
  *              call its first int32 holds the number of boards that were evaluated twice
- * Three launches on `stream`, no synchronisation with the host. */
+ * Two launches on `stream`, no synchronisation with the host, no atomic operation. */
 int c6_cascade_workspace_bytes(int64_t boards, size_t *bytes);
 int c6_forward_cascade(const void *x, int x_dtype, int64_t groups, int64_t boards_per_group,
                        const void *packed, size_t packed_stride, int prec, void *logits, int logits_dtype,

@@ -86,7 +86,8 @@ def test_packed_sizes_follow_the_layout():
     assert _lib.packed_bytes(_lib.PREC_BF16C) == first + _lib.packed_bytes(_lib.PREC_BF16F6W)
     # ... or, for parameters that are exact in bf16, the bf16 + fp6 set
     assert _lib.packed_bytes(_lib.PREC_BF16C6) == first + _lib.packed_bytes(_lib.PREC_BF16F6)
-    assert _lib.cascade_workspace_bytes(0) == 16 and _lib.cascade_workspace_bytes(5) == 48
+    # workspace: 4 ints, 1024 per-run counts, per-run lists with room for boards + 1024 entries
+    assert _lib.cascade_workspace_bytes(0) == 16 + 8192 and _lib.cascade_workspace_bytes(5) == 16 + 8192 + 32
     with pytest.raises(ValueError):
         _lib.packed_bytes(9)
 
@@ -119,7 +120,7 @@ def test_entry_points_reject_bad_arguments_before_touching_the_device():
     assert lib.c6_pack_weights_grouped(None, None, None, None, None, None, 0, 1, None, 0, None) == -1
     size = ctypes.c_size_t(0)
     assert lib.c6_cascade_workspace_bytes(-1, ctypes.byref(size)) == -1
-    assert lib.c6_cascade_workspace_bytes(4096, ctypes.byref(size)) == 0 and size.value == 16 + 4 * 4096
+    assert lib.c6_cascade_workspace_bytes(4096, ctypes.byref(size)) == 0 and size.value == 16 + 8192 + 4 * 4096
     assert lib.c6_mask_logits(None, None, 0, 3, 0, None, None) == -1
     assert lib.c6_mask_logits(None, None, 0, 0, 0, None, None) == 0
     assert lib.c6_softmax_sample(None, None, None, 1.0, 2, None, None, None) == -1
