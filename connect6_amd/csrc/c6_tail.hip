@@ -67,11 +67,14 @@ __global__ void mask_elem_kernel(const T *__restrict__ in, const uint8_t *__rest
 // work on groups of four boards (32 planes for the view gather) and move them with 16-byte
 // accesses; the last, partial group falls back to element accesses.
 
-// Eight boards per group (two per wave): masked softmax over 361 logits and inverse-CDF draw
+// Four boards per group (one per wave): masked softmax over 361 logits and inverse-CDF draw
 // (connect6/train.py:195-213 of the reference, with the uniform supplied).  A workgroup walks
 // over groups; while it works on one group out of LDS, the next group's rows are already on
-// their way into registers, so that every CU always has reads in flight.
-constexpr int kSampleBoards = 8;
+// their way into registers, so that every CU always has reads in flight.  Small groups and many
+// more workgroups than fit the chip at once (each takes about four groups) measured best: eight
+// boards per group on exactly the resident number of workgroups took 118 us for 262,144 boards,
+// this shape 98 us; one group per workgroup, with nothing fetched ahead, 112 us.
+constexpr int kSampleBoards = 4;
 __global__ __launch_bounds__(256) void sample_kernel(const float *__restrict__ logits,
                                                      const uint8_t *__restrict__ legal,
                                                      const float *__restrict__ u,
@@ -81,15 +84,15 @@ __global__ __launch_bounds__(256) void sample_kernel(const float *__restrict__ l
   __shared__ __attribute__((aligned(16))) float s_logit[kSampleBoards * kPix];
   __shared__ __attribute__((aligned(16))) uint8_t s_legal[kSampleBoards * kPix];
   constexpr int NV = kSampleBoards * kPix / 4;       // 16-byte units of a group's logits (722)
-  constexpr int NL = kSampleBoards * kPix / 8;       // 8-byte units of its legality bytes (361)
+  constexpr int NL = kSampleBoards * kPix / 4;       // 4-byte units of its legality bytes (361)
   constexpr int RV = (NV + 255) / 256, RL = (NL + 255) / 256;
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const bool masked = legal != nullptr;
   const bool vec = (reinterpret_cast<uintptr_t>(logits) & 15u) == 0 &&
-                   (!masked || (reinterpret_cast<uintptr_t>(legal) & 7u) == 0);
+                   (!masked || (reinterpret_cast<uintptr_t>(legal) & 3u) == 0);
   const long long groups = (batch + kSampleBoards - 1) / kSampleBoards;
   f32x4 pv[RV];
-  v2i pl[RL];
+  int pl[RL];
   // a full group with aligned operands travels through registers; anything else is copied
   // element by element when its turn comes
   auto prefetch = [&](long long g) {
@@ -104,7 +107,7 @@ __global__ __launch_bounds__(256) void sample_kernel(const float *__restrict__ l
 #pragma unroll
         for (int r = 0; r < RL; ++r) {
           const int i = threadIdx.x + r * 256;
-          if (i < NL) pl[r] = reinterpret_cast<const v2i *>(legal + (size_t)b0 * kPix)[i];
+          if (i < NL) pl[r] = reinterpret_cast<const int *>(legal + (size_t)b0 * kPix)[i];
         }
       }
     }
@@ -124,7 +127,7 @@ __global__ __launch_bounds__(256) void sample_kernel(const float *__restrict__ l
 #pragma unroll
         for (int r = 0; r < RL; ++r) {
           const int i = threadIdx.x + r * 256;
-          if (i < NL) reinterpret_cast<v2i *>(s_legal)[i] = pl[r];
+          if (i < NL) reinterpret_cast<int *>(s_legal)[i] = pl[r];
         }
       }
     } else {
@@ -327,7 +330,7 @@ int launch_mask(const void *logits, const uint8_t *legal, int elem_bytes, long l
 int launch_sample(const float *logits, const uint8_t *legal, const float *u, float inv_t,
                   long long batch, long long *actions, float *logprob, hipStream_t st) {
   const long long groups = (batch + kSampleBoards - 1) / kSampleBoards;
-  const long long resident = 256LL * 8;  // eight workgroups of 256 threads fit a CU; more only queue
+  const long long resident = 256LL * 64;  // (eight workgroups of 256 threads fit a CU at a time; see the kernel)
   hipLaunchKernelGGL(sample_kernel, dim3((unsigned)(groups < resident ? groups : resident)), dim3(256), 0, st, logits,
                      legal, u, inv_t, batch, actions, logprob);
   return check_launch("softmax_sample");
