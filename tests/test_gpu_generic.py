@@ -13,6 +13,11 @@ from tests.util import rel_l2
 pytestmark = pytest.mark.gpu
 
 
+def _lib_prec(dtype):
+    from connect6_amd import _lib
+    return _lib.PREC_F32 if dtype == torch.float32 else _lib.PREC_BF16
+
+
 def test_grouped_history_matches_individual_models_reference_test_shape(cuda):
     # tests/test_training_features.py:120-151 of the reference, on the GPU
     torch.manual_seed(123)
@@ -69,6 +74,18 @@ def test_grouped_generic_is_one_launch_per_layer_and_equals_model_by_model(cuda,
             assert torch.equal(grouped[i], single.to(dtype)), i
             want, _ = R.forward({k: v.to(dtype).float() for k, v in cp.model_state.items()}, x[i].to(dtype).float())
             assert rel_l2(grouped[i].float().cpu(), want) <= (1e-5 if dtype == torch.float32 else 2e-2)
+    # the value head of every weight set too (an ensemble asks for policies only): stacked
+    # parameters of three models through the grouped entry point against model-by-model calls
+    states = [R.init_state(90 + i, "torch_default", kernels=kernels, channels=channels) for i in range(3)]
+    stacked = {k: torch.stack([st[k] for st in states]).to(cuda) for k in states[0]}
+    xs = x[:3].to(cuda)
+    with torch.inference_mode():
+        lg, vg = run_forward_generic(xs.reshape(21, 3, board, board), stacked, kernels, channels, _lib_prec(dtype),
+                                     groups=3, mask_mode=1)
+        for i, st in enumerate(states):
+            l1, v1 = run_forward_generic(xs[i], {k: v.to(cuda) for k, v in st.items()}, kernels, channels,
+                                         _lib_prec(dtype), mask_mode=1)
+            assert torch.equal(lg[7 * i:7 * i + 7], l1) and torch.equal(vg[7 * i:7 * i + 7], v1), i
     # argument checks of the grouped entry point
     import ctypes
 
